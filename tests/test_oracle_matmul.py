@@ -1,0 +1,97 @@
+"""Pins the oracle's two CPU matmuls (ggml-style Q8 activations, and exact)."""
+import numpy as np
+import pytest
+
+import lowbit_oracle as orc
+import np_formats as npf
+
+Q4_0, Q4_1, Q8_0, NF4, FP8 = 2, 3, 8, 10, 15
+ALL = [Q4_0, Q4_1, Q8_0, NF4, FP8]
+
+
+def _case(seed, n, k, m, std=0.02):
+    r = np.random.default_rng(seed)
+    w = (r.standard_normal((n, k)) * std).astype(np.float32)
+    x = r.standard_normal((m, k)).astype(np.float32)
+    return w, x
+
+
+@pytest.mark.parametrize("qtype", ALL)
+def test_exact_is_float64_matmul_of_independent_decode(qtype):
+    w, x = _case(40 + qtype, 48, 256, 3)
+    blob = orc.quantize(w, qtype)
+    wd = npf.DECODERS[qtype](blob, w.shape).astype(np.float64)
+    want = (x.astype(np.float64) @ wd.T).astype(np.float32)
+    got = orc.mul_mat_exact(blob, x, w.shape, qtype)
+    assert got.shape == (3, 48)
+    assert np.array_equal(got, want)
+
+
+def test_hand_computed_q4_0_block():
+    # K = 32, N = 2, M = 1; integer activations with |x|max = 127 quantize to themselves (d = 1)
+    codes = np.array([np.tile(np.arange(16), 2), np.tile(np.arange(15, -1, -1), 2)], dtype=np.uint8)
+    blob = np.zeros((2, 18), dtype=np.uint8)
+    blob[:, :2] = np.array([0.5, -0.25], dtype=np.float16).reshape(2, 1).view(np.uint8)
+    blob[:, 2:] = codes[:, :16] | (codes[:, 16:] << 4)
+    x = np.arange(-16, 16).astype(np.float32)
+    x[0] = 127.0
+    wq = codes.astype(np.int64) - 8
+    want = (wq * x.astype(np.int64)).sum(axis=1) * np.array([0.5, -0.25])
+    got = orc.mul_mat_q(blob.reshape(-1), x.reshape(1, 32), (2, 32), Q4_0)
+    assert np.array_equal(got.ravel(), want.astype(np.float32))
+    assert np.array_equal(orc.mul_mat_exact(blob.reshape(-1), x.reshape(1, 32), (2, 32), Q4_0).ravel(),
+                          want.astype(np.float32))
+
+
+def test_hand_computed_q4_1_and_q8_0_block():
+    x = np.arange(-16, 16).astype(np.float32)
+    x[3] = -127.0
+    xi = x.astype(np.int64)
+    codes = np.tile(np.arange(16), 2).astype(np.uint8)
+    b = np.zeros(20, dtype=np.uint8)
+    b[:2] = np.array([0.25], dtype=np.float16).view(np.uint8)
+    b[2:4] = np.array([-2.0], dtype=np.float16).view(np.uint8)
+    b[4:] = codes[:16] | (codes[16:] << 4)
+    want = 0.25 * (codes.astype(np.int64) * xi).sum() + -2.0 * xi.sum()
+    got = orc.mul_mat_q(b, x.reshape(1, 32), (1, 32), Q4_1)
+    assert got.ravel()[0] == np.float32(want)
+    q = np.arange(-16, 16).astype(np.int8)
+    b = np.zeros(34, dtype=np.uint8)
+    b[:2] = np.array([0.125], dtype=np.float16).view(np.uint8)
+    b[2:] = q.view(np.uint8)
+    want = 0.125 * (q.astype(np.int64) * xi).sum()
+    assert orc.mul_mat_q(b, x.reshape(1, 32), (1, 32), Q8_0).ravel()[0] == np.float32(want)
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("m", [1, 5])
+def test_q_path_stays_close_to_exact(qtype, m):
+    # Q8 activation rounding (step |x|max/127 per block of 32) moves a dot product by about
+    # 0.5 % of max|y|: the reference's own CPU matmul is that far from the exact product, which
+    # is inside the 1e-2 * max|y| parity budget.  nf4 / fp8 use fp32 dequantized weights: tight.
+    w, x = _case(60 + qtype + m, 256, 1024, m)
+    blob = orc.quantize(w, qtype)
+    yq = orc.mul_mat_q(blob, x, w.shape, qtype)
+    ye = orc.mul_mat_exact(blob, x, w.shape, qtype)
+    tol = 8e-3 if qtype in (Q4_0, Q4_1, Q8_0) else 1e-5
+    assert np.abs(yq - ye).max() <= tol * np.abs(ye).max()
+
+
+def test_q_path_matches_numpy_restatement_q4_0():
+    w, x = _case(77, 32, 128, 2)
+    blob = orc.quantize(w, Q4_0)
+    t = blob.reshape(-1, 18)
+    dw = t[:, :2].copy().view(np.float16).astype(np.float32).reshape(32, 4)
+    qw = (np.concatenate([t[:, 2:] & 0xF, t[:, 2:] >> 4], axis=1).astype(np.int32) - 8).reshape(32, 4, 32)
+    xb = x.reshape(2, 4, 32)
+    amax = np.abs(xb).max(axis=-1)
+    d = (amax / np.float32(127.0)).astype(np.float32)
+    inv = (np.float32(1.0) / d).astype(np.float32)
+    qx = npf._roundf((xb * inv[..., None]).astype(np.float32)).astype(np.int32)
+    dx = d.astype(np.float16).astype(np.float32)
+    want = np.zeros((2, 32), dtype=np.float32)
+    for b in range(4):
+        sumi = (qx[:, None, b, :] * qw[None, :, b, :]).sum(axis=-1).astype(np.float32)
+        want = want + (sumi * dw[None, :, b]).astype(np.float32) * dx[:, None, b]
+    got = orc.mul_mat_q(blob, x, w.shape, Q4_0)
+    assert np.array_equal(got, want.astype(np.float32))
