@@ -1,0 +1,124 @@
+/*
+ * C ABI of liblowbit_hip.so: ipex-llm's low-bit linear path on one MI355X.
+ *
+ * Two groups of entry points:
+ *
+ *  (1) the ggml_* symbols that ipex-llm binds with ctypes
+ *      (python/llm/src/ipex_llm/ggml/model/llama/llama_cpp.py:945-1185).  Same
+ *      names, argument order and meaning; all pointers are HOST memory, calls
+ *      are synchronous, buffers are caller-owned.  The work is staged through
+ *      device memory and done by the same kernels as group (2).
+ *
+ *  (2) lowbit_* device entry points for callers that already hold device
+ *      memory: what ipex-llm reaches through the torch ops of xe_linear /
+ *      xe_batch (python/llm/src/ipex_llm/transformers/xpu_ops.py:23-62).  Plain
+ *      device pointers, sizes and a hipStream_t passed as void*; work is
+ *      enqueued on that stream and the call returns without synchronizing.
+ *
+ * Every lowbit_* function returns 0 on success or a negative LOWBIT_E* code;
+ * lowbit_last_error() then describes the failure (thread-local).
+ *
+ * qtype values follow ipex_llm.ggml.quantize.ggml_tensor_qtype
+ * (python/llm/src/ipex_llm/ggml/quantize.py:28-57).
+ */
+#ifndef LOWBIT_ABI_H
+#define LOWBIT_ABI_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LOWBIT_ABI_VERSION 1
+
+/* qtypes */
+#define LOWBIT_QT_SYM_INT4 2   /* ggml Q4_0 */
+#define LOWBIT_QT_ASYM_INT4 3  /* ggml Q4_1 */
+#define LOWBIT_QT_SYM_INT8 8   /* ggml Q8_0 */
+#define LOWBIT_QT_NF4 10
+#define LOWBIT_QT_FP8_E4M3 15
+
+/* weight layouts: GGML = the CPU blob of the reference; TILED = 16x128 tiles for the MFMA
+ * kernels (needs N % 16 == 0 and K % 128 == 0).  Both have the same byte count. */
+#define LOWBIT_LAYOUT_GGML 0
+#define LOWBIT_LAYOUT_TILED 1
+
+/* activation / output element types */
+#define LOWBIT_DT_F16 0
+#define LOWBIT_DT_BF16 1
+#define LOWBIT_DT_F32 2
+
+/* error codes */
+#define LOWBIT_OK 0
+#define LOWBIT_EARG (-1)     /* null / misaligned pointer, negative size */
+#define LOWBIT_EQTYPE (-2)   /* qtype outside {2,3,8,10,15} */
+#define LOWBIT_ESIZE (-3)    /* size too large for one launch */
+#define LOWBIT_EDTYPE (-4)   /* element type not supported by this entry point */
+#define LOWBIT_ESHAPE (-5)   /* K not a multiple of the block, or shape not tileable */
+#define LOWBIT_EHIP (-6)     /* HIP runtime error (no device, launch failure, ...) */
+
+int lowbit_abi_version(void);
+const char *lowbit_last_error(void);
+
+/* ------------------------------------------------------------------ (1) */
+
+/* llama_cpp.py:946-967; called from low_bit_linear.py:162.  n = number of weights, k = row
+ * length.  hist is ignored (the reference never reads it back, low_bit_linear.py:145);
+ * scale_search = true is not implemented and fails.  Returns bytes written, 0 on failure. */
+size_t ggml_quantize_tensor(const float *src, void *dst, int qtype, size_t n, int k, int64_t *hist,
+                            bool scale_search);
+/* llama_cpp.py:1050-1056 and :1059-1065.  0 for a qtype this library does not implement. */
+size_t ggml_type_size(int qtype);
+int ggml_qk_size(int qtype);
+/* llama_cpp.py:1068-1081 and :1084-1099; called from low_bit_linear.py:245,258.
+ * k = number of weights to produce (fp32). */
+void ggml_dequantize_q4_0(const void *src, void *dst, size_t k);
+void ggml_dequantize(const void *src, void *dst, size_t k, int qtype);
+/* llama_cpp.py:1102-1135; called from low_bit_linear.py:203,232.  These carry no row length,
+ * so they cannot build the tiled layout: they copy the blob unchanged, and the result is a
+ * valid device weight in LOWBIT_LAYOUT_GGML (served by the slower any-shape kernels).
+ * Callers that know the shape use lowbit_relayout instead. */
+void ggml_q_format_convet_cpu2xpu(const void *src, void *dst, size_t n, int qtype);
+void ggml_q_format_convet_xpu2cpu(const void *src, void *dst, size_t n, int qtype);
+/* llama_cpp.py:1154-1185; called from low_bit_linear.py:487.  ne = {K, rows} (ggml order),
+ * src0 = ggml blob [N, K], src1 = fp32 [M, K], dst = fp32 [M, N].  Activations are rounded to
+ * fp16 on the device (the reference rounds them to int8 blocks instead). */
+void ggml_compute_forward_mul_mat_q_fp32(const int64_t *src0_ne, const void *src0, int qtype,
+                                         const int64_t *src1_ne, const void *src1, void *dst);
+/* llama_cpp.py:1189-1193.  Selects device 0 and loads the kernels. */
+void llama_init_backend(void);
+
+/* ------------------------------------------------------------------ (2) */
+
+/* Bytes of a blob holding n_weights weights; 0 for an unknown qtype. */
+size_t lowbit_blob_bytes(int qtype, int64_t n_weights);
+/* 1 when [N, K] can be held in LOWBIT_LAYOUT_TILED. */
+int lowbit_tileable(int qtype, int64_t N, int64_t K);
+
+/* ggml_quantize_tensor on device memory: src fp32 [N, K] -> dst blob in `layout`. */
+int lowbit_quantize(const float *src, void *dst, int qtype, int64_t N, int64_t K, int layout, void *stream);
+/* ggml_q_format_convet_cpu2xpu / _xpu2cpu with the shape: src in `src_layout` -> dst in the
+ * other layout.  src and dst must not overlap. */
+int lowbit_relayout(const void *src, void *dst, int qtype, int64_t N, int64_t K, int src_layout, void *stream);
+/* xe_linear.dequant (low_bit_linear.py:534-538) / ggml_dequantize: blob -> dense [N, K]. */
+int lowbit_dequantize(const void *w, void *dst, int qtype, int64_t N, int64_t K, int layout, int out_dtype,
+                      void *stream);
+/* xe_linear.forward_new / xe_batch.batch_forward (low_bit_linear.py:657-668, xpu_ops.py:23-26):
+ * y[M, N] = x[M, K] * dequant(w)[N, K]^T, x and y of act_dtype (f16 or bf16), fp32 accumulation.
+ * Picks the streaming GEMV for small M and the MFMA GEMM for large M. */
+int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                   int64_t N, int64_t K, void *stream);
+/* The two kernels behind lowbit_forward, for callers (and benchmarks) that choose themselves.
+ * waves = 0 lets the library pick the workgroup size of the GEMV. */
+int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                int64_t N, int64_t K, int waves, void *stream);
+int lowbit_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                int64_t N, int64_t K, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

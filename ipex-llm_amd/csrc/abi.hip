@@ -1,0 +1,272 @@
+// extern "C" surface of liblowbit_hip.so (declared in include/lowbit_abi.h).
+#include "../../include/lowbit_abi.h"
+#include "lowbit_formats.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+namespace lowbit {
+int launch_quantize(const float *src, void *dst, int qtype, int64_t N, int64_t K, int layout, hipStream_t st);
+int launch_relayout(const void *src, void *dst, int qtype, int64_t N, int64_t K, int src_layout, hipStream_t st);
+int launch_dequantize(const void *w, void *out, int qtype, int64_t N, int64_t K, int layout, int out_dtype,
+                      hipStream_t st);
+int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
+                int waves, hipStream_t st);
+int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
+                hipStream_t st);
+}  // namespace lowbit
+
+using namespace lowbit;
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static int check_hip(hipError_t e, const char *what) {
+    if (e == hipSuccess) return 0;
+    return fail(LOWBIT_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+static int check_launch(int rc, const char *what) {
+    if (rc == -2) return fail(LOWBIT_EQTYPE, "%s: unsupported qtype", what);
+    if (rc == -3) return fail(LOWBIT_ESIZE, "%s: tensor too large for one launch", what);
+    if (rc == -4) return fail(LOWBIT_EDTYPE, "%s: unsupported element type", what);
+    if (rc == -5) return fail(LOWBIT_ESHAPE, "%s: shape cannot be held in the tiled layout", what);
+    if (rc != 0) return fail(LOWBIT_EARG, "%s: error %d", what, rc);
+    return check_hip(hipGetLastError(), what);
+}
+
+static bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
+
+static int check_weight_shape(const char *what, int qtype, int64_t N, int64_t K, int layout) {
+    const int qk = qk_size(qtype);
+    if (!qk) return fail(LOWBIT_EQTYPE, "%s: unsupported qtype %d", what, qtype);
+    if (N < 0 || K < 0) return fail(LOWBIT_EARG, "%s: negative shape", what);
+    if (K % qk) return fail(LOWBIT_ESHAPE, "%s: K=%lld is not a multiple of the block size %d", what, (long long)K, qk);
+    if (layout != LOWBIT_LAYOUT_GGML && layout != LOWBIT_LAYOUT_TILED)
+        return fail(LOWBIT_EARG, "%s: unknown layout %d", what, layout);
+    if (layout == LOWBIT_LAYOUT_TILED && !lowbit_tileable(qtype, N, K))
+        return fail(LOWBIT_ESHAPE, "%s: [%lld, %lld] needs N %% 16 == 0 and K %% 128 == 0 for the tiled layout", what,
+                    (long long)N, (long long)K);
+    if (N > 0x7fffffff || K > 0x7fffffff) return fail(LOWBIT_ESIZE, "%s: dimension exceeds 2^31", what);
+    return 0;
+}
+
+extern "C" {
+
+int lowbit_abi_version(void) { return LOWBIT_ABI_VERSION; }
+const char *lowbit_last_error(void) { return g_err; }
+
+size_t ggml_type_size(int qtype) { return (size_t)type_size(qtype); }
+int ggml_qk_size(int qtype) { return qk_size(qtype); }
+
+size_t lowbit_blob_bytes(int qtype, int64_t n_weights) {
+    const int qk = qk_size(qtype);
+    if (!qk || n_weights < 0) return 0;
+    return (size_t)(n_weights / qk) * (size_t)type_size(qtype);
+}
+
+int lowbit_tileable(int qtype, int64_t N, int64_t K) {
+    return qk_size(qtype) != 0 && N > 0 && K > 0 && (N % TILE_ROWS) == 0 && (K % TILE_COLS) == 0;
+}
+
+int lowbit_quantize(const float *src, void *dst, int qtype, int64_t N, int64_t K, int layout, void *stream) {
+    if (int rc = check_weight_shape("lowbit_quantize", qtype, N, K, layout)) return rc;
+    if (N * K == 0) return 0;
+    if (!src || !dst || !aligned16(src) || !aligned16(dst))
+        return fail(LOWBIT_EARG, "lowbit_quantize: pointers must be non-null and 16-byte aligned");
+    return check_launch(launch_quantize(src, dst, qtype, N, K, layout, (hipStream_t)stream), "lowbit_quantize");
+}
+
+int lowbit_relayout(const void *src, void *dst, int qtype, int64_t N, int64_t K, int src_layout, void *stream) {
+    if (int rc = check_weight_shape("lowbit_relayout", qtype, N, K, LOWBIT_LAYOUT_TILED)) return rc;
+    if (src_layout != LOWBIT_LAYOUT_GGML && src_layout != LOWBIT_LAYOUT_TILED)
+        return fail(LOWBIT_EARG, "lowbit_relayout: unknown layout %d", src_layout);
+    if (!src || !dst || !aligned16(src) || !aligned16(dst))
+        return fail(LOWBIT_EARG, "lowbit_relayout: pointers must be non-null and 16-byte aligned");
+    const size_t bytes = lowbit_blob_bytes(qtype, N * K);
+    const uintptr_t a = (uintptr_t)src, b = (uintptr_t)dst;
+    if (a < b + bytes && b < a + bytes) return fail(LOWBIT_EARG, "lowbit_relayout: src and dst overlap");
+    return check_launch(launch_relayout(src, dst, qtype, N, K, src_layout, (hipStream_t)stream), "lowbit_relayout");
+}
+
+int lowbit_dequantize(const void *w, void *dst, int qtype, int64_t N, int64_t K, int layout, int out_dtype,
+                      void *stream) {
+    if (int rc = check_weight_shape("lowbit_dequantize", qtype, N, K, layout)) return rc;
+    if (N * K == 0) return 0;
+    if (!w || !dst || !aligned16(w)) return fail(LOWBIT_EARG, "lowbit_dequantize: null or misaligned pointer");
+    return check_launch(launch_dequantize(w, dst, qtype, N, K, layout, out_dtype, (hipStream_t)stream),
+                        "lowbit_dequantize");
+}
+
+static int check_mm(const char *what, const void *x, const void *w, void *y, int qtype, int layout, int act_dtype,
+                    int64_t M, int64_t N, int64_t K) {
+    if (int rc = check_weight_shape(what, qtype, N, K, layout)) return rc;
+    if (M < 0 || M > 0x7fffffff) return fail(LOWBIT_EARG, "%s: bad M", what);
+    if (act_dtype != LOWBIT_DT_F16 && act_dtype != LOWBIT_DT_BF16)
+        return fail(LOWBIT_EDTYPE, "%s: activations must be f16 or bf16", what);
+    if (M * N * K == 0) return 0;
+    if (!x || !w || !y || !aligned16(x) || !aligned16(w) || (((uintptr_t)y) & 1))
+        return fail(LOWBIT_EARG, "%s: null or misaligned pointer (x, w: 16 bytes)", what);
+    if (K % 8) return fail(LOWBIT_ESHAPE, "%s: K must be a multiple of 8", what);
+    return 0;
+}
+
+int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
+                int64_t K, int waves, void *stream) {
+    if (int rc = check_mm("lowbit_gemv", x, w, y, qtype, layout, act_dtype, M, N, K)) return rc;
+    if (M * N == 0) return 0;
+    if (K == 0) return fail(LOWBIT_ESHAPE, "lowbit_gemv: K == 0");
+    return check_launch(launch_gemv(x, w, y, qtype, layout, act_dtype, (int)M, (int)N, (int)K, waves,
+                                    (hipStream_t)stream), "lowbit_gemv");
+}
+
+int lowbit_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
+                int64_t K, void *stream) {
+    if (int rc = check_mm("lowbit_gemm", x, w, y, qtype, layout, act_dtype, M, N, K)) return rc;
+    if (M * N == 0) return 0;
+    if (K == 0) return fail(LOWBIT_ESHAPE, "lowbit_gemm: K == 0");
+    return check_launch(launch_gemm(x, w, y, qtype, layout, act_dtype, (int)M, (int)N, (int)K, (hipStream_t)stream),
+                        "lowbit_gemm");
+}
+
+int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
+                   int64_t K, void *stream) {
+    // The GEMV streams the weights once for up to 16 rows of x; beyond that the MFMA GEMM
+    // (which needs the tiled layout) amortizes the dequantization over a 2-D tile.
+    if (M <= 16 || layout != LOWBIT_LAYOUT_TILED)
+        return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
+    return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------- host-pointer group
+
+namespace {
+
+template <typename T> __global__ void cast_f32_kernel(const float *in, T *out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (T)in[i];
+}
+template <typename T> __global__ void cast_to_f32_kernel(const T *in, float *out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (float)in[i];
+}
+
+struct DevBuf {
+    void *p = nullptr;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+    int alloc(size_t bytes) { return check_hip(hipMalloc(&p, bytes ? bytes : 16), "hipMalloc"); }
+};
+
+int host_dequantize(const void *src, void *dst, size_t k, int qtype) {
+    const int qk = qk_size(qtype);
+    if (!qk) return fail(LOWBIT_EQTYPE, "ggml_dequantize: unsupported qtype %d", qtype);
+    if (k % qk) return fail(LOWBIT_ESHAPE, "ggml_dequantize: k not a multiple of %d", qk);
+    if (k == 0) return 0;
+    const size_t bytes = lowbit_blob_bytes(qtype, (int64_t)k);
+    DevBuf w, o;
+    if (int rc = w.alloc(bytes)) return rc;
+    if (int rc = o.alloc(k * 4)) return rc;
+    if (int rc = check_hip(hipMemcpy(w.p, src, bytes, hipMemcpyHostToDevice), "hipMemcpy")) return rc;
+    // the ggml layout does not depend on the row length: one block per row
+    const int64_t rows = (int64_t)(k / (size_t)qk), cols = qk;
+    if (int rc = lowbit_dequantize(w.p, o.p, qtype, rows, cols, LOWBIT_LAYOUT_GGML, LOWBIT_DT_F32, nullptr)) return rc;
+    return check_hip(hipMemcpy(dst, o.p, k * 4, hipMemcpyDeviceToHost), "hipMemcpy");
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t ggml_quantize_tensor(const float *src, void *dst, int qtype, size_t n, int k, int64_t *hist,
+                            bool scale_search) {
+    (void)hist;
+    g_err[0] = 0;
+    if (scale_search) { fail(LOWBIT_EARG, "ggml_quantize_tensor: scale_search is not implemented"); return 0; }
+    const int qk = qk_size(qtype);
+    if (!qk) { fail(LOWBIT_EQTYPE, "ggml_quantize_tensor: unsupported qtype %d", qtype); return 0; }
+    if (k <= 0 || k % qk || n % (size_t)k) { fail(LOWBIT_ESHAPE, "ggml_quantize_tensor: bad n/k"); return 0; }
+    if (n == 0) return 0;
+    const size_t bytes = lowbit_blob_bytes(qtype, (int64_t)n);
+    DevBuf s, d;
+    if (s.alloc(n * 4) || d.alloc(bytes)) return 0;
+    if (check_hip(hipMemcpy(s.p, src, n * 4, hipMemcpyHostToDevice), "hipMemcpy")) return 0;
+    if (lowbit_quantize((const float *)s.p, d.p, qtype, (int64_t)(n / (size_t)k), k, LOWBIT_LAYOUT_GGML, nullptr)) return 0;
+    if (check_hip(hipMemcpy(dst, d.p, bytes, hipMemcpyDeviceToHost), "hipMemcpy")) return 0;
+    return bytes;
+}
+
+void ggml_dequantize_q4_0(const void *src, void *dst, size_t k) {
+    g_err[0] = 0;
+    (void)host_dequantize(src, dst, k, LOWBIT_QT_SYM_INT4);
+}
+
+void ggml_dequantize(const void *src, void *dst, size_t k, int qtype) {
+    g_err[0] = 0;
+    (void)host_dequantize(src, dst, k, qtype);
+}
+
+void ggml_q_format_convet_cpu2xpu(const void *src, void *dst, size_t n, int qtype) {
+    g_err[0] = 0;
+    const size_t bytes = lowbit_blob_bytes(qtype, (int64_t)n);
+    if (!bytes && n) { fail(LOWBIT_EQTYPE, "ggml_q_format_convet_cpu2xpu: unsupported qtype %d", qtype); return; }
+    if (src != dst) memmove(dst, src, bytes);
+}
+
+void ggml_q_format_convet_xpu2cpu(const void *src, void *dst, size_t n, int qtype) {
+    g_err[0] = 0;
+    const size_t bytes = lowbit_blob_bytes(qtype, (int64_t)n);
+    if (!bytes && n) { fail(LOWBIT_EQTYPE, "ggml_q_format_convet_xpu2cpu: unsupported qtype %d", qtype); return; }
+    if (src != dst) memmove(dst, src, bytes);
+}
+
+void ggml_compute_forward_mul_mat_q_fp32(const int64_t *src0_ne, const void *src0, int qtype, const int64_t *src1_ne,
+                                         const void *src1, void *dst) {
+    g_err[0] = 0;
+    const int64_t K = src0_ne[0], N = src0_ne[1], M = src1_ne[1];
+    if (src1_ne[0] != K) { fail(LOWBIT_ESHAPE, "mul_mat: inner dimensions differ"); return; }
+    if (check_weight_shape("ggml_compute_forward_mul_mat_q_fp32", qtype, N, K, LOWBIT_LAYOUT_GGML)) return;
+    if (M * N == 0) return;
+    const size_t wbytes = lowbit_blob_bytes(qtype, N * K);
+    const bool tile = lowbit_tileable(qtype, N, K);
+    DevBuf w, wt, xf, xh, yh, yf;
+    if (w.alloc(wbytes) || xf.alloc((size_t)M * K * 4) || xh.alloc((size_t)M * K * 2) ||
+        yh.alloc((size_t)M * N * 2) || yf.alloc((size_t)M * N * 4)) return;
+    if (tile && wt.alloc(wbytes)) return;
+    if (check_hip(hipMemcpy(w.p, src0, wbytes, hipMemcpyHostToDevice), "hipMemcpy")) return;
+    if (check_hip(hipMemcpy(xf.p, src1, (size_t)M * K * 4, hipMemcpyHostToDevice), "hipMemcpy")) return;
+    const int64_t nx = M * K, ny = M * N;
+    hipLaunchKernelGGL((cast_f32_kernel<_Float16>), dim3((unsigned)((nx + 255) / 256)), dim3(256), 0, nullptr,
+                       (const float *)xf.p, (_Float16 *)xh.p, nx);
+    const void *wdev = w.p;
+    int layout = LOWBIT_LAYOUT_GGML;
+    if (tile) {
+        if (lowbit_relayout(w.p, wt.p, qtype, N, K, LOWBIT_LAYOUT_GGML, nullptr)) return;
+        wdev = wt.p;
+        layout = LOWBIT_LAYOUT_TILED;
+    }
+    if (lowbit_forward(xh.p, wdev, yh.p, qtype, layout, LOWBIT_DT_F16, M, N, K, nullptr)) return;
+    hipLaunchKernelGGL((cast_to_f32_kernel<_Float16>), dim3((unsigned)((ny + 255) / 256)), dim3(256), 0, nullptr,
+                       (const _Float16 *)yh.p, (float *)yf.p, ny);
+    if (check_hip(hipGetLastError(), "cast")) return;
+    (void)check_hip(hipMemcpy(dst, yf.p, (size_t)ny * 4, hipMemcpyDeviceToHost), "hipMemcpy");
+}
+
+void llama_init_backend(void) {
+    g_err[0] = 0;
+    int n = 0;
+    if (check_hip(hipGetDeviceCount(&n), "hipGetDeviceCount")) return;
+    if (n < 1) { fail(LOWBIT_EHIP, "llama_init_backend: no HIP device"); return; }
+    (void)check_hip(hipSetDevice(0), "hipSetDevice");
+}
+
+}  // extern "C"

@@ -1,0 +1,132 @@
+// Layout conversion (ggml <-> tiled) and full dequantization.
+//
+// relayout replaces ggml_q_format_convet_cpu2xpu / _xpu2cpu
+// (python/llm/src/ipex_llm/transformers/low_bit_linear.py:178-233); dequantize
+// replaces ggml_dequantize / ggml_dequantize_q4_0 (low_bit_linear.py:236-259)
+// and xe_linear.dequant (low_bit_linear.py:534-538).  Both are one-off,
+// HBM-bound passes: one thread moves one 32-column sub-block.
+#include "lowbit_formats.h"
+
+namespace lowbit {
+
+template <int QT, int SRC_LAYOUT>
+__global__ __launch_bounds__(256) void relayout_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                       int64_t N, int64_t K) {
+    using F = Fmt<QT>;
+    constexpr int SPB = F::QK / 32;
+    const int64_t sbpr = K / 32;                               // sub-blocks per row
+    if constexpr (QT == QT_NF4 && SRC_LAYOUT == LAYOUT_TILED) {
+        // a ggml nf4 byte mixes both halves of a 64-block: one thread moves a whole block
+        const int64_t blk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (blk >= N * (K / 64)) return;
+        const int64_t n = blk / (K / 64);
+        const int kb = (int)(blk % (K / 64));
+        SubBlock a, b;
+        tiled_load_sub<QT>(src, n, K, kb * 2, a);
+        tiled_load_sub<QT>(src, n, K, kb * 2 + 1, b);
+        uint8_t code64[64];
+        for (int i = 0; i < 32; i++) { code64[i] = a.code[i]; code64[32 + i] = b.code[i]; }
+        ggml_store_nf4_block(dst, blk, code64, a.hdr);
+    } else {
+        const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (t >= N * sbpr) return;
+        const int64_t n = t / sbpr;
+        const int sb = (int)(t % sbpr);
+        SubBlock s;
+        if constexpr (SRC_LAYOUT == LAYOUT_GGML) {
+            ggml_load_sub<QT>(src, n, K, sb, s);
+            tiled_store_codes<QT>(dst, n, K, sb, s.code);
+            if (sb % SPB == 0) tiled_store_hdr<QT>(dst, n, K, sb, s.hdr);
+        } else {
+            tiled_load_sub<QT>(src, n, K, sb, s);
+            ggml_store_sub<QT>(dst, n, K, sb, s.code, s.hdr);
+        }
+    }
+}
+
+template <int QT> static int launch_rl(const void *src, void *dst, int64_t N, int64_t K, int src_layout, hipStream_t st) {
+    int64_t threads = N * (K / 32);
+    if (QT == QT_NF4 && src_layout == LAYOUT_TILED) threads = N * (K / 64);
+    if (threads == 0) return 0;
+    const int64_t grid = (threads + 255) / 256;
+    if (grid > 0x7fffffff) return -3;
+    if (src_layout == LAYOUT_GGML)
+        hipLaunchKernelGGL((relayout_kernel<QT, LAYOUT_GGML>), dim3((unsigned)grid), dim3(256), 0, st,
+                           (const uint8_t *)src, (uint8_t *)dst, N, K);
+    else
+        hipLaunchKernelGGL((relayout_kernel<QT, LAYOUT_TILED>), dim3((unsigned)grid), dim3(256), 0, st,
+                           (const uint8_t *)src, (uint8_t *)dst, N, K);
+    return 0;
+}
+
+int launch_relayout(const void *src, void *dst, int qtype, int64_t N, int64_t K, int src_layout, hipStream_t st) {
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_rl<QT_SYM_INT4>(src, dst, N, K, src_layout, st);
+    case QT_ASYM_INT4: return launch_rl<QT_ASYM_INT4>(src, dst, N, K, src_layout, st);
+    case QT_SYM_INT8: return launch_rl<QT_SYM_INT8>(src, dst, N, K, src_layout, st);
+    case QT_NF4: return launch_rl<QT_NF4>(src, dst, N, K, src_layout, st);
+    case QT_FP8_E4M3: return launch_rl<QT_FP8_E4M3>(src, dst, N, K, src_layout, st);
+    default: return -2;
+    }
+}
+
+// ------------------------------------------------------------ dequantize
+
+template <typename T> __device__ inline T from_f32(float v);
+template <> __device__ inline float from_f32<float>(float v) { return v; }
+template <> __device__ inline _Float16 from_f32<_Float16>(float v) { return (_Float16)v; }
+template <> __device__ inline __bf16 from_f32<__bf16>(float v) { return (__bf16)v; }
+
+template <int QT, int LAYOUT, typename OT>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict__ w, OT *__restrict__ out,
+                                                      int64_t N, int64_t K) {
+    const int64_t sbpr = K / 32;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= N * sbpr) return;
+    const int64_t n = t / sbpr;
+    const int sb = (int)(t % sbpr);
+    SubBlock s;
+    if constexpr (LAYOUT == LAYOUT_GGML) ggml_load_sub<QT>(w, n, K, sb, s);
+    else tiled_load_sub<QT>(w, n, K, sb, s);
+    OT *o = out + n * K + (int64_t)sb * 32;
+#pragma unroll
+    for (int i = 0; i < 32; i++) o[i] = from_f32<OT>(decode<QT>(s.code[i], s.d, s.m));
+}
+
+template <int QT, typename OT>
+static int launch_dq2(const void *w, void *out, int64_t N, int64_t K, int layout, hipStream_t st) {
+    const int64_t threads = N * (K / 32);
+    if (threads == 0) return 0;
+    const int64_t grid = (threads + 255) / 256;
+    if (grid > 0x7fffffff) return -3;
+    if (layout == LAYOUT_GGML)
+        hipLaunchKernelGGL((dequant_kernel<QT, LAYOUT_GGML, OT>), dim3((unsigned)grid), dim3(256), 0, st,
+                           (const uint8_t *)w, (OT *)out, N, K);
+    else
+        hipLaunchKernelGGL((dequant_kernel<QT, LAYOUT_TILED, OT>), dim3((unsigned)grid), dim3(256), 0, st,
+                           (const uint8_t *)w, (OT *)out, N, K);
+    return 0;
+}
+
+template <int QT> static int launch_dq(const void *w, void *out, int64_t N, int64_t K, int layout, int dt, hipStream_t st) {
+    switch (dt) {
+    case DT_F16: return launch_dq2<QT, _Float16>(w, out, N, K, layout, st);
+    case DT_BF16: return launch_dq2<QT, __bf16>(w, out, N, K, layout, st);
+    case DT_F32: return launch_dq2<QT, float>(w, out, N, K, layout, st);
+    default: return -4;
+    }
+}
+
+int launch_dequantize(const void *w, void *out, int qtype, int64_t N, int64_t K, int layout, int out_dtype,
+                      hipStream_t st) {
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_dq<QT_SYM_INT4>(w, out, N, K, layout, out_dtype, st);
+    case QT_ASYM_INT4: return launch_dq<QT_ASYM_INT4>(w, out, N, K, layout, out_dtype, st);
+    case QT_SYM_INT8: return launch_dq<QT_SYM_INT8>(w, out, N, K, layout, out_dtype, st);
+    case QT_NF4: return launch_dq<QT_NF4>(w, out, N, K, layout, out_dtype, st);
+    case QT_FP8_E4M3: return launch_dq<QT_FP8_E4M3>(w, out, N, K, layout, out_dtype, st);
+    default: return -2;
+    }
+}
+
+}  // namespace lowbit

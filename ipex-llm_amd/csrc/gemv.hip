@@ -1,0 +1,358 @@
+// Decode-time product y[M,N] = x[M,K] * dequant(W)[N,K]^T for small M.
+//
+// Replaces xe_linear.forward_new at M = 1 and xe_batch.batch_forward at small M
+// (python/llm/src/ipex_llm/transformers/low_bit_linear.py:657-668).
+//
+// gemv_mfma_kernel (tiled layout): HBM-bound streaming of the packed weights.
+//   One workgroup owns one tile row (16 output columns) and its waves split
+//   the 128-column tiles along K.  A lane's 16-byte load of a tile is already
+//   its B operand for four v_mfma_f32_16x16x32 (one per 32-column sub-block);
+//   codes are turned into exact small numbers in registers (never scaled in
+//   half precision), the activations are the A operand (rows = batch index),
+//   and the block scale is applied to the fp32 MFMA result.  M <= 16 costs the
+//   same weight traffic as M = 1.  Algorithmic bytes per launch:
+//   N*K*TS/QK (weights) + M*K*2 (x) + M*N*2 (y).
+// gemv_generic_kernel: any layout / any shape fallback, one wave per row.
+#include "lowbit_formats.h"
+
+namespace lowbit {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename AT> struct Vec8;
+template <> struct Vec8<_Float16> { typedef f16x8 type; };
+template <> struct Vec8<__bf16> { typedef bf16x8 type; };
+
+__device__ inline f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+__device__ inline f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+
+template <typename AT> __device__ inline AT to_at(float v);
+template <> __device__ inline _Float16 to_at<_Float16>(float v) { return (_Float16)v; }
+template <> __device__ inline __bf16 to_at<__bf16>(float v) { return (__bf16)v; }
+
+__device__ inline uint32_t and_or(uint32_t a, uint32_t b, uint32_t c) { return (a & b) | c; }
+
+// ---- codes of one sub-block (8 columns of this lane) -> B operand ----------
+//
+// The operand holds the *unscaled* code value (q - 8, q, int8, e4m3 value, nf4
+// code-book entry); OFFSET<> says what constant is still folded in and has to
+// be removed with the row sum of x (0 for every path below except bf16 4-bit).
+
+template <int QT, typename AT> struct Unpack;
+
+// 4-bit integer codes, fp16: 0x6400 | q is the half 1024 + q; 0x6400 | q << 4 is 1024 + 16 q.
+template <> struct Unpack<QT_SYM_INT4, _Float16> {
+    static constexpr float OFFSET = 0.0f;
+    __device__ static f16x8 run(uint32_t v, const void *) {
+        const f16x2 k1032 = {(_Float16)1032.0f, (_Float16)1032.0f};
+        const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
+        const f16x2 k72 = {(_Float16)72.0f, (_Float16)72.0f};
+        const uint32_t v8 = v >> 8;
+        f16x2 t0 = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1032;
+        f16x2 t1 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k72);
+        f16x2 t2 = __builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, 0x64006400u)) - k1032;
+        f16x2 t3 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, 0x64006400u)), k16th, -k72);
+        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+    }
+};
+template <> struct Unpack<QT_ASYM_INT4, _Float16> {
+    static constexpr float OFFSET = 0.0f;
+    __device__ static f16x8 run(uint32_t v, const void *) {
+        const f16x2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+        const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
+        const f16x2 k64 = {(_Float16)64.0f, (_Float16)64.0f};
+        const uint32_t v8 = v >> 8;
+        f16x2 t0 = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1024;
+        f16x2 t1 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k64);
+        f16x2 t2 = __builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, 0x64006400u)) - k1024;
+        f16x2 t3 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, 0x64006400u)), k16th, -k64);
+        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+    }
+};
+// 4-bit integer codes, bf16: 0x4300 | q is the bf16 128 + q (exact); the constant is removed
+// afterwards through the row sum of x, which a second MFMA against all-ones provides.
+template <int QT> struct UnpackInt4Bf16 {
+    static constexpr float OFFSET = (QT == QT_SYM_INT4) ? 136.0f : 128.0f;
+    __device__ static bf16x8 run(uint32_t v, const void *) {
+        u32x4 t;
+        t[0] = and_or(v, 0x000f000fu, 0x43004300u);
+        t[1] = and_or(v >> 4, 0x000f000fu, 0x43004300u);
+        t[2] = and_or(v >> 8, 0x000f000fu, 0x43004300u);
+        t[3] = and_or(v >> 12, 0x000f000fu, 0x43004300u);
+        return __builtin_bit_cast(bf16x8, t);
+    }
+};
+template <> struct Unpack<QT_SYM_INT4, __bf16> : UnpackInt4Bf16<QT_SYM_INT4> {};
+template <> struct Unpack<QT_ASYM_INT4, __bf16> : UnpackInt4Bf16<QT_ASYM_INT4> {};
+
+// nf4: code-book lookup from a 16-entry table in LDS (entries already in the activation type).
+template <typename AT> struct Unpack<QT_NF4, AT> {
+    static constexpr float OFFSET = 0.0f;
+    __device__ static typename Vec8<AT>::type run(uint32_t v, const void *lut_) {
+        const AT *lut = (const AT *)lut_;
+        typename Vec8<AT>::type r;
+        r[0] = lut[v & 0xf]; r[2] = lut[(v >> 4) & 0xf]; r[4] = lut[(v >> 8) & 0xf]; r[6] = lut[(v >> 12) & 0xf];
+        r[1] = lut[(v >> 16) & 0xf]; r[3] = lut[(v >> 20) & 0xf]; r[5] = lut[(v >> 24) & 0xf]; r[7] = lut[v >> 28];
+        return r;
+    }
+};
+
+// 8-bit codes: two dwords (columns 0..3, 4..7).
+template <int QT, typename AT> struct Unpack8;
+template <> struct Unpack8<QT_SYM_INT8, _Float16> {
+    __device__ static f16x8 run(uint32_t lo, uint32_t hi) {
+        // byte ^ 0x80 = q + 128 (unsigned); 0x6400 | u is the half 1024 + u
+        const f16x2 k1152 = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const uint32_t a = lo ^ 0x80808080u, b = hi ^ 0x80808080u;
+        const uint32_t c64 = 0x64646464u;
+        f16x2 t0 = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, a, 0x04010400u)) - k1152;
+        f16x2 t1 = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, a, 0x04030402u)) - k1152;
+        f16x2 t2 = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, b, 0x04010400u)) - k1152;
+        f16x2 t3 = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, b, 0x04030402u)) - k1152;
+        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+    }
+};
+template <> struct Unpack8<QT_SYM_INT8, __bf16> {
+    __device__ static bf16x8 run(uint32_t lo, uint32_t hi) {
+        bf16x8 r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            r[i] = (__bf16)(float)(int8_t)(lo >> (8 * i));      // |q| <= 128: exact in bf16
+            r[4 + i] = (__bf16)(float)(int8_t)(hi >> (8 * i));
+        }
+        return r;
+    }
+};
+template <> struct Unpack8<QT_FP8_E4M3, _Float16> {
+    __device__ static f16x8 run(uint32_t lo, uint32_t hi) {
+        f16x2 t0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false);
+        f16x2 t1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true);
+        f16x2 t2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false);
+        f16x2 t3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true);
+        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+    }
+};
+template <> struct Unpack8<QT_FP8_E4M3, __bf16> {
+    __device__ static bf16x8 run(uint32_t lo, uint32_t hi) {
+        bf16x2 t0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+        bf16x2 t1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+        bf16x2 t2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+        bf16x2 t3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+        return bf16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+    }
+};
+
+template <int QT, typename AT> constexpr float code_offset() {
+    if constexpr (Fmt<QT>::BITS == 4) return Unpack<QT, AT>::OFFSET;
+    else return 0.0f;
+}
+
+template <typename AT> __device__ inline typename Vec8<AT>::type ones8() {
+    typename Vec8<AT>::type r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r[i] = to_at<AT>(1.0f);
+    return r;
+}
+
+// ------------------------------------------------------------ MFMA GEMV
+
+constexpr int GEMV_MAX_WAVES = 16;
+
+template <int QT, typename AT, int MT>
+__global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+                                                         AT *__restrict__ y, int M, int N, int K) {
+    using F = Fmt<QT>;
+    using V8 = typename Vec8<AT>::type;
+    constexpr bool IS4 = (F::BITS == 4);
+    constexpr bool ASYM = (QT == QT_ASYM_INT4);
+    constexpr float OFFSET = code_offset<QT, AT>();
+    constexpr bool NEED_S = ASYM || OFFSET != 0.0f;
+
+    __shared__ float red[GEMV_MAX_WAVES][MT][64];
+    __shared__ AT lut[16];
+    if constexpr (QT == QT_NF4) {
+        if (threadIdx.x < 16) lut[threadIdx.x] = to_at<AT>(NF4_CODEBOOK[threadIdx.x]);
+        __syncthreads();
+    }
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, W = blockDim.x >> 6;
+    const int G = K / TILE_COLS;
+    const int r = lane & 15, c = lane >> 4;
+    // A rows: row r carries batch index (r/4)*MT + r%4 when r%4 < MT, so that the C registers
+    // i < MT of lane group g hold batch indices g*MT + i and nothing else has to be scaled.
+    const int m_of_r = (r >> 2) * MT + (r & 3);
+    const bool a_valid = ((r & 3) < MT) && (m_of_r < M);
+    const AT *xrow = x + (int64_t)(a_valid ? m_of_r : 0) * K + 8 * c;
+    const uint8_t *wrow = w + (int64_t)blockIdx.x * G * F::TILE_BYTES;
+
+    float acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+    const V8 ones = ones8<AT>();
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int g = wave; g < G; g += W) {
+        const uint8_t *tile = wrow + (int64_t)g * F::TILE_BYTES;
+        u32x4 q0 = *(const u32x4 *)(tile + lane * 16);
+        u32x4 q1 = {0, 0, 0, 0};
+        if constexpr (!IS4) q1 = *(const u32x4 *)(tile + 1024 + lane * 16);
+
+        // headers of this lane's row (r is also the tile row of the B operand)
+        float d[4], mm[4];
+        if constexpr (QT == QT_SYM_INT4 || QT == QT_SYM_INT8) {
+            const u32x2 h = *(const u32x2 *)(tile + F::TILE_CODE_BYTES + r * 8);
+            d[0] = h2f(h[0] & 0xffff); d[1] = h2f(h[0] >> 16); d[2] = h2f(h[1] & 0xffff); d[3] = h2f(h[1] >> 16);
+        } else if constexpr (QT == QT_ASYM_INT4) {
+            const u32x4 h = *(const u32x4 *)(tile + F::TILE_CODE_BYTES + r * 16);
+#pragma unroll
+            for (int j = 0; j < 4; j++) { d[j] = h2f(h[j] & 0xffff); mm[j] = h2f(h[j] >> 16); }
+        } else if constexpr (QT == QT_NF4) {
+            const uint32_t h = *(const uint32_t *)(tile + F::TILE_CODE_BYTES + r * 4);
+            d[0] = d[1] = h2f(h & 0xffff); d[2] = d[3] = h2f(h >> 16);
+        } else {
+            const float s = *(const float *)(tile + F::TILE_CODE_BYTES + r * 4);
+            d[0] = d[1] = d[2] = d[3] = s;
+        }
+
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            V8 a;
+            if (a_valid) a = *(const V8 *)(xrow + (int64_t)(g * 4 + j) * 32);
+            else a = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
+            V8 b;
+            if constexpr (IS4) b = Unpack<QT, AT>::run(q0[j], lut);
+            else if (j < 2) b = Unpack8<QT, AT>::run(q0[2 * j], q0[2 * j + 1]);
+            else b = Unpack8<QT, AT>::run(q1[2 * (j - 2)], q1[2 * (j - 2) + 1]);
+            const f32x4 p = mfma16(a, b, zero4);
+            if constexpr (NEED_S) {
+                const f32x4 s = mfma16(a, ones, zero4);
+                const float e = (ASYM ? mm[j] : 0.0f) - OFFSET * d[j];
+#pragma unroll
+                for (int i = 0; i < MT; i++) acc[i] = fmaf(e, s[i], fmaf(d[j], p[i], acc[i]));
+            } else {
+#pragma unroll
+                for (int i = 0; i < MT; i++) acc[i] = fmaf(d[j], p[i], acc[i]);
+            }
+        }
+    }
+
+    // sum the K-slices of the waves; wave 0 writes.  C layout: lane = 16*grp + col, register i = row 4*grp + i.
+#pragma unroll
+    for (int i = 0; i < MT; i++) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    if (wave == 0) {
+        const int grp = lane >> 4, col = lane & 15;
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float s = 0.0f;
+            for (int ww = 0; ww < W; ww++) s += red[ww][i][lane];
+            const int m = grp * MT + i;
+            if (m < M) y[(int64_t)m * N + (int64_t)blockIdx.x * 16 + col] = to_at<AT>(s);
+        }
+    }
+}
+
+// --------------------------------------------------------- generic GEMV
+
+template <int QT, int LAYOUT, typename AT, int MC>
+__global__ __launch_bounds__(256) void gemv_generic_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+                                                           AT *__restrict__ y, int m0, int M, int N, int K) {
+    const int lane = threadIdx.x & 63;
+    const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    float acc[MC];
+#pragma unroll
+    for (int i = 0; i < MC; i++) acc[i] = 0.0f;
+    const int sbpr = K / 32;
+    for (int sb = lane; sb < sbpr; sb += 64) {
+        SubBlock s;
+        if constexpr (LAYOUT == LAYOUT_GGML) ggml_load_sub<QT>(w, n, K, sb, s);
+        else tiled_load_sub<QT>(w, n, K, sb, s);
+        float wv[32];
+#pragma unroll
+        for (int i = 0; i < 32; i++) wv[i] = decode<QT>(s.code[i], s.d, s.m);
+#pragma unroll
+        for (int mi = 0; mi < MC; mi++) {
+            if (m0 + mi < M) {
+                const AT *xp = x + (int64_t)(m0 + mi) * K + sb * 32;
+                float a = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 32; i++) a = fmaf((float)xp[i], wv[i], a);
+                acc[mi] += a;
+            }
+        }
+    }
+#pragma unroll
+    for (int mi = 0; mi < MC; mi++) {
+        float v = acc[mi];
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        if (lane == 0 && m0 + mi < M) y[(int64_t)(m0 + mi) * N + n] = to_at<AT>(v);
+    }
+}
+
+// -------------------------------------------------------------- launch
+
+static int pick_waves(int G) {
+    // enough waves that each streams about 4 tiles, capped by the block size limit
+    int wv = (G + 3) / 4;
+    if (wv < 1) wv = 1;
+    if (wv > GEMV_MAX_WAVES) wv = GEMV_MAX_WAVES;
+    return wv;
+}
+
+template <int QT, typename AT>
+static int launch_gemv_t(const void *x, const void *w, void *y, int layout, int M, int N, int K, int waves,
+                         hipStream_t st) {
+    const bool tiled_ok = layout == LAYOUT_TILED && (N % TILE_ROWS) == 0 && (K % TILE_COLS) == 0;
+    if (layout == LAYOUT_TILED && !tiled_ok) return -5;
+    if (tiled_ok) {
+        const int G = K / TILE_COLS;
+        const int wv = waves > 0 ? (waves > GEMV_MAX_WAVES ? GEMV_MAX_WAVES : waves) : pick_waves(G);
+        for (int m0 = 0; m0 < M; m0 += 16) {
+            const int mc = (M - m0) < 16 ? (M - m0) : 16;
+            const AT *xp = (const AT *)x + (int64_t)m0 * K;
+            AT *yp = (AT *)y + (int64_t)m0 * N;
+            dim3 grid(N / TILE_ROWS), block(64 * wv);
+            if (mc <= 4)
+                hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, 1>), grid, block, 0, st, xp, (const uint8_t *)w, yp, mc, N, K);
+            else if (mc <= 8)
+                hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, 2>), grid, block, 0, st, xp, (const uint8_t *)w, yp, mc, N, K);
+            else
+                hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, 4>), grid, block, 0, st, xp, (const uint8_t *)w, yp, mc, N, K);
+        }
+        return 0;
+    }
+    for (int m0 = 0; m0 < M; m0 += 4)
+        hipLaunchKernelGGL((gemv_generic_kernel<QT, LAYOUT_GGML, AT, 4>), dim3((N + 3) / 4), dim3(256), 0, st,
+                           (const AT *)x, (const uint8_t *)w, (AT *)y, m0, M, N, K);
+    return 0;
+}
+
+template <int QT>
+static int launch_gemv_q(const void *x, const void *w, void *y, int layout, int dt, int M, int N, int K, int waves,
+                         hipStream_t st) {
+    if (dt == DT_F16) return launch_gemv_t<QT, _Float16>(x, w, y, layout, M, N, K, waves, st);
+    if (dt == DT_BF16) return launch_gemv_t<QT, __bf16>(x, w, y, layout, M, N, K, waves, st);
+    return -4;
+}
+
+int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
+                int waves, hipStream_t st) {
+    if (M == 0 || N == 0) return 0;
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_gemv_q<QT_SYM_INT4>(x, w, y, layout, act_dtype, M, N, K, waves, st);
+    case QT_ASYM_INT4: return launch_gemv_q<QT_ASYM_INT4>(x, w, y, layout, act_dtype, M, N, K, waves, st);
+    case QT_SYM_INT8: return launch_gemv_q<QT_SYM_INT8>(x, w, y, layout, act_dtype, M, N, K, waves, st);
+    case QT_NF4: return launch_gemv_q<QT_NF4>(x, w, y, layout, act_dtype, M, N, K, waves, st);
+    case QT_FP8_E4M3: return launch_gemv_q<QT_FP8_E4M3>(x, w, y, layout, act_dtype, M, N, K, waves, st);
+    default: return -2;
+    }
+}
+
+}  // namespace lowbit

@@ -1,0 +1,211 @@
+"""ctypes binding of liblowbit_hip.so.
+
+Takes the place of the reference module of the same name
+(python/llm/src/ipex_llm/ggml/model/llama/llama_cpp.py:71-109 for the loader,
+:945-1185 for the ggml_* prototypes).  The ggml_* functions keep their
+signatures; the lowbit_* functions are the device-pointer entry points that
+stand where the reference calls the xe_linear / xe_batch torch ops.
+
+There is no CPU implementation behind this module: if the HIP library cannot
+be loaded, importing it raises RuntimeError, exactly as the reference does when
+libllama-api.so is missing.
+"""
+import ctypes
+import os
+import pathlib
+
+from ipex_llm.utils.common import invalidInputError
+from ipex_llm.utils.utils import get_shared_lib_info
+
+LAYOUT_GGML = 0
+LAYOUT_TILED = 1
+DT_F16, DT_BF16, DT_F32 = 0, 1, 2
+
+
+def _load_shared_library(lib_base_name: str):
+    _base_path, _lib_paths = get_shared_lib_info(lib_base_name=lib_base_name)
+    if "LLAMA_CPP_LIB" in os.environ:
+        _lib = pathlib.Path(os.environ["LLAMA_CPP_LIB"])
+        _lib_paths = [_lib.resolve()]
+    for _lib_path in _lib_paths:
+        if _lib_path.exists():
+            try:
+                return ctypes.CDLL(str(_lib_path))
+            except Exception as e:  # noqa: BLE001
+                invalidInputError(False, f"Failed to load shared library '{_lib_path}': {e}.")
+    invalidInputError(False,
+                      f"Shared library with base name '{lib_base_name}' not found "
+                      f"(looked for {[str(p) for p in _lib_paths]}); build it with "
+                      "`make -C ipex-llm_amd/csrc`. There is no CPU fallback.")
+
+
+_lib_base_name = "lowbit_hip"
+_lib = _load_shared_library(_lib_base_name)
+
+c_void_p, c_int, c_int64, c_size_t = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
+
+_lib.lowbit_abi_version.argtypes = []
+_lib.lowbit_abi_version.restype = c_int
+_lib.lowbit_last_error.argtypes = []
+_lib.lowbit_last_error.restype = ctypes.c_char_p
+
+
+def last_error() -> str:
+    return (_lib.lowbit_last_error() or b"").decode("utf-8", "replace")
+
+
+def _check(rc: int, what: str):
+    invalidInputError(rc == 0, f"{what} failed ({rc}): {last_error()}")
+
+
+def _check_void(what: str):
+    msg = last_error()
+    invalidInputError(msg == "", f"{what} failed: {msg}")
+
+
+# ------------------------------------------------------------------ ggml_* (host pointers)
+
+_lib.ggml_quantize_tensor.argtypes = [ctypes.POINTER(ctypes.c_float), c_void_p, c_int, c_size_t, c_int,
+                                      ctypes.POINTER(c_int64), ctypes.c_bool]
+_lib.ggml_quantize_tensor.restype = c_size_t
+
+
+def ggml_quantize_tensor(src, dst, qtype, n, k, hist, scale_search) -> int:
+    written = _lib.ggml_quantize_tensor(src, dst, qtype, n, k, hist, scale_search)
+    if n:
+        _check_void("ggml_quantize_tensor")
+    return written
+
+
+def _unsupported(name):
+    def f(*args, **kwargs):
+        invalidInputError(False, f"{name} is not provided by the MI355X low-bit library "
+                                 "(k-quant / NPU round-to-nearest quantizers are outside its scope).")
+    f.__name__ = name
+    return f
+
+
+ggml_quantize_tensor_with_weights = _unsupported("ggml_quantize_tensor_with_weights")
+ggml_quantize_tensor_rtn = _unsupported("ggml_quantize_tensor_rtn")
+ggml_quantize_tensor_rtn_with_weights = _unsupported("ggml_quantize_tensor_rtn_with_weights")
+
+_lib.ggml_type_size.argtypes = [c_int]
+_lib.ggml_type_size.restype = c_size_t
+_lib.ggml_qk_size.argtypes = [c_int]
+_lib.ggml_qk_size.restype = c_int
+
+
+def ggml_type_size(qtype) -> int:
+    return _lib.ggml_type_size(qtype)
+
+
+def ggml_qk_size(qtype) -> int:
+    return _lib.ggml_qk_size(qtype)
+
+
+_lib.ggml_dequantize_q4_0.argtypes = [c_void_p, c_void_p, c_size_t]
+_lib.ggml_dequantize_q4_0.restype = None
+_lib.ggml_dequantize.argtypes = [c_void_p, c_void_p, c_size_t, c_int]
+_lib.ggml_dequantize.restype = None
+
+
+def ggml_dequantize_q4_0(src, dst, k):
+    _lib.ggml_dequantize_q4_0(src, dst, k)
+    _check_void("ggml_dequantize_q4_0")
+
+
+def ggml_dequantize(src, dst, k, qtype):
+    _lib.ggml_dequantize(src, dst, k, qtype)
+    _check_void("ggml_dequantize")
+
+
+_lib.ggml_q_format_convet_cpu2xpu.argtypes = [c_void_p, c_void_p, c_size_t, c_int]
+_lib.ggml_q_format_convet_cpu2xpu.restype = None
+_lib.ggml_q_format_convet_xpu2cpu.argtypes = [c_void_p, c_void_p, c_size_t, c_int]
+_lib.ggml_q_format_convet_xpu2cpu.restype = None
+
+
+def ggml_q_format_convet_cpu2xpu(src, dst, n, qtype):
+    _lib.ggml_q_format_convet_cpu2xpu(src, dst, n, qtype)
+    _check_void("ggml_q_format_convet_cpu2xpu")
+
+
+def ggml_q_format_convet_xpu2cpu(src, dst, n, qtype):
+    _lib.ggml_q_format_convet_xpu2cpu(src, dst, n, qtype)
+    _check_void("ggml_q_format_convet_xpu2cpu")
+
+
+_lib.ggml_compute_forward_mul_mat_q_fp32.argtypes = [ctypes.POINTER(c_int64), c_void_p, c_int,
+                                                     ctypes.POINTER(c_int64), c_void_p, c_void_p]
+_lib.ggml_compute_forward_mul_mat_q_fp32.restype = None
+
+
+def ggml_compute_forward_mul_mat_q_fp32(src_0_ne, src_0_data, src_0_qtype, src_1_ne, src_1_data, result):
+    _lib.ggml_compute_forward_mul_mat_q_fp32(src_0_ne, src_0_data, src_0_qtype, src_1_ne, src_1_data, result)
+    _check_void("ggml_compute_forward_mul_mat_q_fp32")
+
+
+_lib.llama_init_backend.argtypes = []
+_lib.llama_init_backend.restype = None
+
+
+def llama_init_backend():
+    _lib.llama_init_backend()
+
+
+# ---------------------------------------------------------------- lowbit_* (device pointers)
+
+_lib.lowbit_blob_bytes.argtypes = [c_int, c_int64]
+_lib.lowbit_blob_bytes.restype = c_size_t
+_lib.lowbit_tileable.argtypes = [c_int, c_int64, c_int64]
+_lib.lowbit_tileable.restype = c_int
+_lib.lowbit_quantize.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p]
+_lib.lowbit_quantize.restype = c_int
+_lib.lowbit_relayout.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p]
+_lib.lowbit_relayout.restype = c_int
+_lib.lowbit_dequantize.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p]
+_lib.lowbit_dequantize.restype = c_int
+_lib.lowbit_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
+                                c_void_p]
+_lib.lowbit_forward.restype = c_int
+_lib.lowbit_gemv.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
+                             c_int, c_void_p]
+_lib.lowbit_gemv.restype = c_int
+_lib.lowbit_gemm.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
+                             c_void_p]
+_lib.lowbit_gemm.restype = c_int
+
+
+def lowbit_blob_bytes(qtype, n_weights) -> int:
+    return _lib.lowbit_blob_bytes(qtype, n_weights)
+
+
+def lowbit_tileable(qtype, n, k) -> bool:
+    return bool(_lib.lowbit_tileable(qtype, n, k))
+
+
+def lowbit_quantize(src, dst, qtype, n, k, layout, stream):
+    _check(_lib.lowbit_quantize(src, dst, qtype, n, k, layout, stream), "lowbit_quantize")
+
+
+def lowbit_relayout(src, dst, qtype, n, k, src_layout, stream):
+    _check(_lib.lowbit_relayout(src, dst, qtype, n, k, src_layout, stream), "lowbit_relayout")
+
+
+def lowbit_dequantize(w, dst, qtype, n, k, layout, out_dtype, stream):
+    _check(_lib.lowbit_dequantize(w, dst, qtype, n, k, layout, out_dtype, stream), "lowbit_dequantize")
+
+
+def lowbit_forward(x, w, y, qtype, layout, act_dtype, m, n, k, stream):
+    _check(_lib.lowbit_forward(x, w, y, qtype, layout, act_dtype, m, n, k, stream), "lowbit_forward")
+
+
+def lowbit_gemv(x, w, y, qtype, layout, act_dtype, m, n, k, waves, stream):
+    _check(_lib.lowbit_gemv(x, w, y, qtype, layout, act_dtype, m, n, k, waves, stream), "lowbit_gemv")
+
+
+def lowbit_gemm(x, w, y, qtype, layout, act_dtype, m, n, k, stream):
+    _check(_lib.lowbit_gemm(x, w, y, qtype, layout, act_dtype, m, n, k, stream), "lowbit_gemm")
+
+
+llama_init_backend()

@@ -1,0 +1,166 @@
+"""HIP path against the CPU oracle, through the C ABI, on a real MI355X."""
+import numpy as np
+import pytest
+import torch
+
+import lowbit_oracle as orc
+from gpu_util import (ALL, FP8, NF4, Q4_0, Q4_1, Q8_0, acts, dev_dequantize, dev_matmul, dev_quantize,
+                      dev_relayout, weights)
+
+pytestmark = pytest.mark.gpu
+
+GGML, TILED = 0, 1
+
+
+# ------------------------------------------------------------------ quantizer: bit exact
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("shape", [(16, 128), (64, 512), (3, 128), (272, 1408), (1024, 4096)])
+def test_quantize_bytes_match_oracle(qtype, shape):
+    w = weights(1000 + qtype + shape[0], shape)
+    got = dev_quantize(w, qtype, GGML).cpu().numpy()
+    want = orc.quantize(w, qtype)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("qtype", ALL)
+def test_quantize_edge_blocks(qtype):
+    qk = orc.qk_size(qtype)
+    rows = []
+    rows.append(np.zeros(qk))                                   # all zero
+    rows.append(np.full(qk, 0.75))                              # constant
+    r = np.random.default_rng(5)
+    a = r.standard_normal(qk) * 0.02
+    a[3], a[qk - 2] = 0.4, -0.4                                 # +max first, same |.| later
+    rows.append(a)
+    b = a.copy()
+    b[3], b[qk - 2] = -0.4, 0.4
+    rows.append(b)
+    rows.append(np.tile(np.arange(-8, 8), qk // 16) * 0.125)    # exact ramp
+    rows.append(r.standard_normal(qk) * 1e-7)                   # tiny: fp16 subnormal scale
+    rows.append(r.standard_normal(qk) * 3e4)                    # huge: scale near fp16 max
+    c = np.zeros(qk)
+    c[0] = 1.0
+    c[1:9] = (np.arange(8) + 0.5) / 8.0                         # exact .5 ties for sym_int4
+    rows.append(c)
+    w = np.stack(rows).astype(np.float32)
+    got = dev_quantize(w, qtype, GGML).cpu().numpy()
+    assert np.array_equal(got, orc.quantize(w, qtype))
+
+
+@pytest.mark.parametrize("qtype", ALL)
+def test_tiled_quantize_equals_relayout_and_round_trips(qtype):
+    n, k = 48, 640
+    w = weights(2000 + qtype, (n, k))
+    g = dev_quantize(w, qtype, GGML)
+    t = dev_quantize(w, qtype, TILED)
+    t2 = dev_relayout(g, qtype, n, k, GGML)
+    assert torch.equal(t, t2)
+    assert not torch.equal(t, g)
+    back = dev_relayout(t, qtype, n, k, TILED)
+    assert torch.equal(back, g)
+    assert np.array_equal(back.cpu().numpy(), orc.quantize(w, qtype))
+
+
+# ---------------------------------------------------------------- dequantizer
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("layout", [GGML, TILED])
+def test_dequantize_fp32_bit_exact(qtype, layout):
+    n, k = 32, 512
+    w = weights(3000 + qtype, (n, k))
+    blob = dev_quantize(w, qtype, layout)
+    got = dev_dequantize(blob, qtype, n, k, layout, torch.float32).cpu().numpy()
+    want = orc.dequantize(orc.quantize(w, qtype), qtype, (n, k))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_dequantize_half_types_are_rounded_fp32(qtype, dtype):
+    n, k = 16, 256
+    w = weights(3100 + qtype, (n, k))
+    blob = dev_quantize(w, qtype, TILED)
+    got = dev_dequantize(blob, qtype, n, k, TILED, dtype).cpu()
+    want = torch.from_numpy(orc.dequantize(orc.quantize(w, qtype), qtype, (n, k))).to(dtype)
+    assert torch.equal(got, want)
+
+
+# -------------------------------------------------------------------- matmul
+
+def _tol(dtype, qtype):
+    # output rounding (2^-11 / 2^-8 of |y|) plus accumulation order; nf4 in bf16 also rounds its
+    # code book to 8 bits.  All far inside the 1e-2 * max|y| budget of the parity bar.
+    if dtype == torch.float16:
+        return 1.5e-3
+    return 8e-3 if qtype == NF4 else 6e-3
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 2, 4, 5, 8, 9, 16])
+def test_gemv_tiled_against_oracle(qtype, dtype, m):
+    n, k = 96, 1024
+    w = weights(4000 + qtype, (n, k))
+    x = acts(4100 + m, m, k, dtype)
+    blob_np = orc.quantize(w, qtype)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n, fn="gemv")
+    xf = x.float().numpy()
+    y_exact = orc.mul_mat_exact(blob_np, xf, (n, k), qtype)
+    y_ref = orc.mul_mat_q(blob_np, xf, (n, k), qtype)       # the reference's CPU low-bit matmul
+    assert np.isfinite(y).all()
+    assert np.abs(y - y_exact).max() <= _tol(dtype, qtype) * np.abs(y_exact).max()
+    assert np.abs(y - y_ref).max() <= 1e-2 * np.abs(y_ref).max()
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("waves", [1, 3, 16])
+def test_gemv_any_wave_count(qtype, waves):
+    n, k = 32, 896      # 7 tiles along K: uneven split over the waves
+    w = weights(4200 + qtype, (n, k))
+    x = acts(4300, 3, k, torch.float16)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n, fn="gemv", waves=waves)
+    y_exact = orc.mul_mat_exact(orc.quantize(w, qtype), x.float().numpy(), (n, k), qtype)
+    assert np.abs(y - y_exact).max() <= 1.5e-3 * np.abs(y_exact).max()
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_generic_kernel_on_untileable_shapes(qtype, dtype):
+    qk = orc.qk_size(qtype)
+    n, k = 37, qk * 3
+    w = weights(4400 + qtype, (n, k))
+    x = acts(4500, 5, k, dtype)
+    blob = dev_quantize(w, qtype, GGML)
+    y = dev_matmul(x, blob, qtype, GGML, n)
+    y_exact = orc.mul_mat_exact(orc.quantize(w, qtype), x.float().numpy(), (n, k), qtype)
+    assert np.abs(y - y_exact).max() <= _tol(dtype, qtype) * np.abs(y_exact).max()
+
+
+@pytest.mark.parametrize("qtype", ALL)
+def test_forward_m_above_16(qtype):
+    n, k = 64, 512
+    w = weights(4600 + qtype, (n, k))
+    x = acts(4700, 40, k, torch.float16)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n)
+    y_exact = orc.mul_mat_exact(orc.quantize(w, qtype), x.float().numpy(), (n, k), qtype)
+    assert np.abs(y - y_exact).max() <= 1.5e-3 * np.abs(y_exact).max()
+
+
+def test_headline_shape_sym_int4_m1():
+    # BASELINE configs[0]: [4096, 4096] sym_int4, M = 1, fp16
+    n = k = 4096
+    w = weights(1001, (n, k), outliers=False)
+    x = acts(1002, 1, k, torch.float16)
+    blob = dev_quantize(w, Q4_0, TILED)
+    blob_np = orc.quantize(w, Q4_0)
+    assert np.array_equal(dev_relayout(blob, Q4_0, n, k, TILED).cpu().numpy(), blob_np)
+    y = dev_matmul(x, blob, Q4_0, TILED, n)
+    xf = x.float().numpy()
+    y_exact = orc.mul_mat_exact(blob_np, xf, (n, k), Q4_0)
+    y_ref = orc.mul_mat_q(blob_np, xf, (n, k), Q4_0)
+    assert np.abs(y - y_exact).max() <= 1.5e-3 * np.abs(y_exact).max()
+    assert np.abs(y - y_ref).max() <= 1e-2 * np.abs(y_ref).max()
