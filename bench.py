@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Benchmark of the low-bit linear hot path on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input: the
+Llama-2-7B decode linear sweep of BASELINE.json configs[1] - 32 layers x
+(q, k, v, o [4096x4096], gate, up [11008x4096], down [4096x11008]) in sym_int4,
+fp16 activations at M = 1, every linear a separate dependent launch.  The 224
+launches of a sweep are captured once in a HIP graph and replayed, so that
+Python launch cost is not billed as bandwidth.  Weights (3.64 GB) are resident
+in HBM before the timed region and exceed the 256 MB Infinity Cache, so every
+sweep streams them from HBM.
+
+Prints ONE JSON line (see README / DESIGN.md for the fields).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "ipex-llm_amd"))
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16/bf16 MFMA peak
+
+SYM_INT4 = 2
+LLAMA2_7B = [("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
+             ("gate", 11008, 4096), ("up", 11008, 4096), ("down", 4096, 11008)]
+N_LAYERS = 32
+
+
+def blob_bytes(n, k):
+    return n * k // 32 * 18
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--m", type=int, default=1, help="rows of x (decode batch)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the M=4/8 and single-shape figures")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no sharding, no collectives); --gpus must be 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the low-bit kernels have no CPU implementation", file=sys.stderr)
+        sys.exit(3)
+    import ipex_llm.ggml.model.llama.llama_cpp as ggml
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1002)
+
+    def stream():
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    # ---- synthetic weights: N(0, 0.02) with 0.1 % outliers at +-0.5, quantized on the GPU
+    layers = []
+    for _ in range(N_LAYERS):
+        mods = []
+        for name, n, k in LLAMA2_7B:
+            w = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
+            mask = torch.rand((n, k), generator=gen, device=dev) < 0.001
+            sign = torch.where(torch.rand((n, k), generator=gen, device=dev) < 0.5, 0.5, -0.5)
+            w = torch.where(mask, sign, w)
+            blob = torch.empty(blob_bytes(n, k), dtype=torch.uint8, device=dev)
+            ggml.lowbit_quantize(w.data_ptr(), blob.data_ptr(), SYM_INT4, n, k, ggml.LAYOUT_TILED, stream())
+            mods.append((name, n, k, blob))
+            del w, mask, sign
+        layers.append(mods)
+    torch.cuda.synchronize()
+
+    def make_io(m):
+        xs = {k: torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32).half()
+              for k in (4096, 11008)}
+        ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for n in (4096, 11008)}
+        return xs, ys
+
+    def sweep(m, xs, ys):
+        st = stream()
+        for mods in layers:
+            for _, n, k, blob in mods:
+                ggml.lowbit_forward(xs[k].data_ptr(), blob.data_ptr(), ys[n].data_ptr(), SYM_INT4,
+                                    ggml.LAYOUT_TILED, ggml.DT_F16, m, n, k, st)
+
+    def capture(fn):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()                                   # eager warm-up on the capture stream
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g
+
+    def time_graph(g, steps, warmup):
+        for _ in range(warmup):
+            g.replay()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps         # ms per replay
+
+    launches = N_LAYERS * len(LLAMA2_7B)
+    w_bytes = sum(blob_bytes(n, k) for _, n, k in LLAMA2_7B) * N_LAYERS
+
+    def sweep_bytes(m):
+        io = sum(m * k * 2 + m * n * 2 for _, n, k in LLAMA2_7B) * N_LAYERS
+        return w_bytes + io
+
+    xs, ys = make_io(args.m)
+    g = capture(lambda: sweep(args.m, xs, ys))
+    ms = time_graph(g, args.steps, args.warmup)
+    total = sweep_bytes(args.m)
+    gbs = total / (ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "sym_int4 decode GEMV GB/s",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "Llama-2-7B decode linear sweep (BASELINE configs[1]): 32 layers x 7 "
+                               "linears, sym_int4, fp16 x, one launch per linear, HIP-graph replay",
+                   "M": args.m, "launches_per_step": launches, "weight_bytes_per_step": w_bytes,
+                   "algorithmic_bytes_per_step": total},
+        "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+    }
+    # dominant kernel = the streaming GEMV (one symbol for all 7 shapes); a launch processes on
+    # average 1/224 of the sweep's algorithmic bytes
+    per_launch = total / launches
+    avg_us = ms * 1e3 / launches
+    out["roofline"] = {"bound": "hbm", "kernel": "gemv_mfma_kernel<sym_int4,f16>",
+                       "achieved": round(per_launch / (avg_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                       "unit": "GB/s", "frac": round(per_launch / (avg_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                       "traffic": None, "bytes_per_launch": round(per_launch), "avg_launch_us": round(avg_us, 3)}
+
+    if not args.no_extra:
+        extra = {}
+        for m in (4, 8):
+            if m == args.m:
+                continue
+            xs2, ys2 = make_io(m)
+            g2 = capture(lambda: sweep(m, xs2, ys2))
+            ms2 = time_graph(g2, max(5, args.steps // 2), 3)
+            extra[f"sweep_M{m}"] = {"ms_per_step": round(ms2, 4),
+                                    "GB/s": round(sweep_bytes(m) / (ms2 * 1e-3) / 1e9, 1)}
+            del g2
+        # the metric's single shape, K=4096 N=11008, cycling over the 64 distinct gate/up weights
+        # (1.6 GB, far beyond the Infinity Cache)
+        gu = [b for mods in layers for (name, n, k, b) in mods if name in ("gate", "up")]
+
+        def headline():
+            st = stream()
+            for b in gu:
+                ggml.lowbit_forward(xs[4096].data_ptr(), b.data_ptr(), ys[11008].data_ptr(), SYM_INT4,
+                                    ggml.LAYOUT_TILED, ggml.DT_F16, args.m, 11008, 4096, st)
+        g3 = capture(headline)
+        ms3 = time_graph(g3, max(5, args.steps // 2), 3)
+        hb = blob_bytes(11008, 4096) + args.m * 4096 * 2 + args.m * 11008 * 2
+        us = ms3 * 1e3 / len(gu)
+        extra["gemv_N11008_K4096"] = {"us_per_launch": round(us, 3), "GB/s": round(hb / (us * 1e-6) / 1e9, 1),
+                                      "pct_hbm_peak": round(100 * hb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 2),
+                                      "algorithmic_bytes": hb}
+        # prefill: one [11008 x 4096] linear at M = 2048
+        m = 2048
+        xp = torch.randn((m, 4096), generator=gen, device=dev, dtype=torch.float32).half()
+        yp = torch.empty((m, 11008), dtype=torch.float16, device=dev)
+
+        def prefill():
+            st = stream()
+            for b in gu[:8]:
+                ggml.lowbit_forward(xp.data_ptr(), b.data_ptr(), yp.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED,
+                                    ggml.DT_F16, m, 11008, 4096, st)
+        g4 = capture(prefill)
+        ms4 = time_graph(g4, 5, 2) / 8
+        flop = 2.0 * m * 11008 * 4096
+        extra["prefill_M2048_N11008_K4096"] = {"ms": round(ms4, 4), "TFLOP/s": round(flop / (ms4 * 1e-3) / 1e12, 1),
+                                               "pct_f16_mfma_peak": round(100 * flop / (ms4 * 1e-3) / 1e12 /
+                                                                          MFMA_F16_PEAK_TFLOPS, 2)}
+        out["extra"] = extra
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(layers[0], args.m, ggml, torch)
+
+    print(json.dumps(out))
+
+
+def cpu_baseline(mods, m, ggml, torch):
+    """The reference's CPU low-bit matmul (restated in oracle/) on the host cores, on a bounded
+    sample: the 7 linears of ONE layer, repeated for about 10 s."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import lowbit_oracle as orc
+    threads = orc.max_threads()
+    blobs = []
+    for name, n, k, blob in mods:
+        g = torch.empty_like(blob)
+        ggml.lowbit_relayout(blob.data_ptr(), g.data_ptr(), SYM_INT4, n, k, ggml.LAYOUT_TILED,
+                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        blobs.append((n, k, g.cpu().numpy()))
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(7)
+    xs = {k: rng.standard_normal((m, k)).astype(np.float32) for k in (4096, 11008)}
+    nbytes = sum(b.size + m * k * 2 + m * n * 2 for n, k, b in blobs)
+
+    def one_pass():
+        for n, k, b in blobs:
+            orc.mul_mat_q(b, xs[k], (n, k), SYM_INT4)
+    one_pass()
+    t0 = time.perf_counter()
+    passes = 0
+    while True:
+        one_pass()
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt > 10.0 or passes >= 200:
+            break
+    return {"value": round(nbytes * passes / dt / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"1 of 32 layers (7 linears, {nbytes} algorithmic bytes) x {passes} passes, "
+                      f"oracle ggml-style Q8_0-activation matmul, OpenMP"}
+
+
+if __name__ == "__main__":
+    main()
