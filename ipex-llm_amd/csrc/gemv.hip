@@ -163,8 +163,49 @@ template <typename AT> __device__ inline typename Vec8<AT>::type ones8() {
 // ------------------------------------------------------------ MFMA GEMV
 
 constexpr int GEMV_MAX_WAVES = 16;
+constexpr int GEMV_LDS_X_BUDGET = 64 * 1024;
 
-template <int QT, typename AT, int MT>
+// Raw tile registers of one lane: codes (16 or 32 bytes) and the headers of its row.
+template <int QT> struct TileRegs {
+    u32x4 q0, q1;
+    u32x4 h;
+};
+
+template <int QT> __device__ inline void load_tile(const uint8_t *tile, int lane, int r, TileRegs<QT> &t) {
+    using F = Fmt<QT>;
+    t.q0 = *(const u32x4 *)(tile + lane * 16);
+    if constexpr (F::BITS == 8) t.q1 = *(const u32x4 *)(tile + 1024 + lane * 16);
+    if constexpr (QT == QT_SYM_INT4 || QT == QT_SYM_INT8) {
+        const u32x2 h = *(const u32x2 *)(tile + F::TILE_CODE_BYTES + r * 8);
+        t.h[0] = h[0]; t.h[1] = h[1];
+    } else if constexpr (QT == QT_ASYM_INT4) {
+        t.h = *(const u32x4 *)(tile + F::TILE_CODE_BYTES + r * 16);
+    } else {
+        t.h[0] = *(const uint32_t *)(tile + F::TILE_CODE_BYTES + r * 4);
+    }
+}
+
+// scale (and minimum) of sub-block j of the lane's row
+template <int QT> __device__ inline void tile_scale(const TileRegs<QT> &t, int j, float &d, float &m) {
+    m = 0.0f;
+    if constexpr (QT == QT_SYM_INT4 || QT == QT_SYM_INT8) {
+        const uint32_t h = t.h[j >> 1];
+        d = h2f((j & 1) ? (h >> 16) : (h & 0xffff));
+    } else if constexpr (QT == QT_ASYM_INT4) {
+        d = h2f(t.h[j] & 0xffff);
+        m = h2f(t.h[j] >> 16);
+    } else if constexpr (QT == QT_NF4) {
+        d = h2f((j >> 1) ? (t.h[0] >> 16) : (t.h[0] & 0xffff));
+    } else {
+        d = __builtin_bit_cast(float, t.h[0]);
+    }
+}
+
+// One workgroup = one tile row (16 output columns).  Per round, wave w owns U consecutive
+// tiles along K: it first issues every weight load of the round (so the whole slice is in
+// flight at once), then copies its slice of x into a wave-private LDS region, then runs
+// 4*U MFMAs whose A operand comes from LDS.  Rounds repeat until K is covered.
+template <int QT, typename AT, int MT, int U, int XN>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                          AT *__restrict__ y, int M, int N, int K) {
     using F = Fmt<QT>;
@@ -173,7 +214,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     constexpr bool ASYM = (QT == QT_ASYM_INT4);
     constexpr float OFFSET = code_offset<QT, AT>();
     constexpr bool NEED_S = ASYM || OFFSET != 0.0f;
+    constexpr int SLICE = U * TILE_COLS;                    // columns of x per wave and round
 
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float red[GEMV_MAX_WAVES][MT][64];
     __shared__ AT lut[16];
     if constexpr (QT == QT_NF4) {
@@ -186,10 +229,13 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     const int r = lane & 15, c = lane >> 4;
     // A rows: row r carries batch index (r/4)*MT + r%4 when r%4 < MT, so that the C registers
     // i < MT of lane group g hold batch indices g*MT + i and nothing else has to be scaled.
-    const int m_of_r = (r >> 2) * MT + (r & 3);
-    const bool a_valid = ((r & 3) < MT) && (m_of_r < M);
-    const AT *xrow = x + (int64_t)(a_valid ? m_of_r : 0) * K + 8 * c;
+    // Rows with r%4 >= MT (and batch indices >= M) only feed C rows that are never read, so
+    // they may hold anything: they re-read a valid row, which LDS serves as a broadcast.
+    int m_of_r = (r >> 2) * MT + ((r & 3) < MT ? (r & 3) : MT - 1);
+    m_of_r = m_of_r < M ? m_of_r : M - 1;
     const uint8_t *wrow = w + (int64_t)blockIdx.x * G * F::TILE_BYTES;
+    AT *xs = (AT *)smem + (int64_t)wave * (XN * 512);       // [XN*64/(SLICE/8)][SLICE], private to this wave
+    const AT *xa = xs + m_of_r * SLICE + 8 * c;
 
     float acc[MT];
 #pragma unroll
@@ -197,47 +243,68 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     const V8 ones = ones8<AT>();
     const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
-    for (int g = wave; g < G; g += W) {
-        const uint8_t *tile = wrow + (int64_t)g * F::TILE_BYTES;
-        u32x4 q0 = *(const u32x4 *)(tile + lane * 16);
-        u32x4 q1 = {0, 0, 0, 0};
-        if constexpr (!IS4) q1 = *(const u32x4 *)(tile + 1024 + lane * 16);
-
-        // headers of this lane's row (r is also the tile row of the B operand)
-        float d[4], mm[4];
-        if constexpr (QT == QT_SYM_INT4 || QT == QT_SYM_INT8) {
-            const u32x2 h = *(const u32x2 *)(tile + F::TILE_CODE_BYTES + r * 8);
-            d[0] = h2f(h[0] & 0xffff); d[1] = h2f(h[0] >> 16); d[2] = h2f(h[1] & 0xffff); d[3] = h2f(h[1] >> 16);
-        } else if constexpr (QT == QT_ASYM_INT4) {
-            const u32x4 h = *(const u32x4 *)(tile + F::TILE_CODE_BYTES + r * 16);
+    for (int g0 = 0; g0 < G; g0 += W * U) {
+        const int gw = g0 + wave * U;
+        // Straight-line loads (addresses clamped instead of branches, so that the compiler can
+        // count outstanding loads): x first - it comes from L2 and is needed before any MFMA -
+        // then every weight tile of the round.  Loads return in order, so the LDS copy of x
+        // waits for the x loads only and each tile is consumed as soon as it lands while the
+        // later ones are still in flight.  XN = 16-byte chunks of x per lane (>= M*U/4).
+        u32x4 xv[XN];
 #pragma unroll
-            for (int j = 0; j < 4; j++) { d[j] = h2f(h[j] & 0xffff); mm[j] = h2f(h[j] >> 16); }
-        } else if constexpr (QT == QT_NF4) {
-            const uint32_t h = *(const uint32_t *)(tile + F::TILE_CODE_BYTES + r * 4);
-            d[0] = d[1] = h2f(h & 0xffff); d[2] = d[3] = h2f(h >> 16);
-        } else {
-            const float s = *(const float *)(tile + F::TILE_CODE_BYTES + r * 4);
-            d[0] = d[1] = d[2] = d[3] = s;
+        for (int i = 0; i < XN; i++) {
+            const int idx = i * 64 + lane;
+            int m = idx / (SLICE / 8);
+            const int u = idx % (SLICE / 8);
+            int col = gw * TILE_COLS + u * 8;
+            m = m < M ? m : M - 1;
+            col = col < K ? col : K - 8;                    // out-of-range tiles carry a zero scale
+            xv[i] = *(const u32x4 *)(x + (int64_t)m * K + col);
+        }
+        __builtin_amdgcn_sched_barrier(0);                  // keep the x loads ahead of the weight loads
+        TileRegs<QT> tr[U];
+#pragma unroll
+        for (int t = 0; t < U; t++) {
+            const int g = gw + t;
+            load_tile<QT>(wrow + (int64_t)(g < G ? g : G - 1) * F::TILE_BYTES, lane, r, tr[t]);
         }
 
+        __builtin_amdgcn_sched_barrier(0);
+        // The LDS region is private to the wave and LDS operations of a wave execute in order:
+        // a wavefront-scope fence (no hardware wait) is all the synchronization it needs.
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            V8 a;
-            if (a_valid) a = *(const V8 *)(xrow + (int64_t)(g * 4 + j) * 32);
-            else a = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
-            V8 b;
-            if constexpr (IS4) b = Unpack<QT, AT>::run(q0[j], lut);
-            else if (j < 2) b = Unpack8<QT, AT>::run(q0[2 * j], q0[2 * j + 1]);
-            else b = Unpack8<QT, AT>::run(q1[2 * (j - 2)], q1[2 * (j - 2) + 1]);
-            const f32x4 p = mfma16(a, b, zero4);
-            if constexpr (NEED_S) {
-                const f32x4 s = mfma16(a, ones, zero4);
-                const float e = (ASYM ? mm[j] : 0.0f) - OFFSET * d[j];
+        for (int i = 0; i < XN; i++) *(u32x4 *)(xs + (i * 64 + lane) * 8) = xv[i];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+
 #pragma unroll
-                for (int i = 0; i < MT; i++) acc[i] = fmaf(e, s[i], fmaf(d[j], p[i], acc[i]));
-            } else {
+        for (int t = 0; t < U; t++) {
+            const bool live = gw + t < G;
+            V8 a[4];
 #pragma unroll
-                for (int i = 0; i < MT; i++) acc[i] = fmaf(d[j], p[i], acc[i]);
+            for (int j = 0; j < 4; j++) a[j] = *(const V8 *)(xa + (t * 4 + j) * 32);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                V8 b;
+                if constexpr (IS4) b = Unpack<QT, AT>::run(tr[t].q0[j], lut);
+                else if (j < 2) b = Unpack8<QT, AT>::run(tr[t].q0[2 * j], tr[t].q0[2 * j + 1]);
+                else b = Unpack8<QT, AT>::run(tr[t].q1[2 * (j - 2)], tr[t].q1[2 * (j - 2) + 1]);
+                float d, mn;
+                tile_scale<QT>(tr[t], j, d, mn);
+                d = live ? d : 0.0f;
+                mn = live ? mn : 0.0f;
+                const f32x4 p = mfma16(a[j], b, zero4);
+                if constexpr (NEED_S) {
+                    const f32x4 s = mfma16(a[j], ones, zero4);
+                    const float e = mn - OFFSET * d;
+#pragma unroll
+                    for (int i = 0; i < MT; i++) acc[i] = fmaf(e, s[i], fmaf(d, p[i], acc[i]));
+                } else {
+#pragma unroll
+                    for (int i = 0; i < MT; i++) acc[i] = fmaf(d, p[i], acc[i]);
+                }
             }
         }
     }
@@ -298,12 +365,19 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const AT *__restrict_
 
 // -------------------------------------------------------------- launch
 
-static int pick_waves(int G) {
-    // enough waves that each streams about 4 tiles, capped by the block size limit
-    int wv = (G + 3) / 4;
-    if (wv < 1) wv = 1;
+template <int QT, typename AT, int MT, int U, int XN>
+static void launch_mfma(const AT *x, const uint8_t *w, AT *y, int M, int N, int K, int waves, hipStream_t st) {
+    const int G = K / TILE_COLS;
+    // waves: enough that one round covers K, within the block size limit and the LDS budget for x
+    int wv = (G + U - 1) / U;
+    const int lds_cap = GEMV_LDS_X_BUDGET / (XN * 512 * (int)sizeof(AT));
+    if (wv > lds_cap) wv = lds_cap;
     if (wv > GEMV_MAX_WAVES) wv = GEMV_MAX_WAVES;
-    return wv;
+    if (waves > 0 && waves < wv) wv = waves;
+    if (wv < 1) wv = 1;
+    const size_t lds = (size_t)wv * XN * 512 * sizeof(AT);
+    hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, MT, U, XN>), dim3(N / TILE_ROWS), dim3(64 * wv), lds, st, x, w, y, M, N,
+                       K);
 }
 
 template <int QT, typename AT>
@@ -312,19 +386,15 @@ static int launch_gemv_t(const void *x, const void *w, void *y, int layout, int 
     const bool tiled_ok = layout == LAYOUT_TILED && (N % TILE_ROWS) == 0 && (K % TILE_COLS) == 0;
     if (layout == LAYOUT_TILED && !tiled_ok) return -5;
     if (tiled_ok) {
-        const int G = K / TILE_COLS;
-        const int wv = waves > 0 ? (waves > GEMV_MAX_WAVES ? GEMV_MAX_WAVES : waves) : pick_waves(G);
         for (int m0 = 0; m0 < M; m0 += 16) {
             const int mc = (M - m0) < 16 ? (M - m0) : 16;
             const AT *xp = (const AT *)x + (int64_t)m0 * K;
             AT *yp = (AT *)y + (int64_t)m0 * N;
-            dim3 grid(N / TILE_ROWS), block(64 * wv);
-            if (mc <= 4)
-                hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, 1>), grid, block, 0, st, xp, (const uint8_t *)w, yp, mc, N, K);
-            else if (mc <= 8)
-                hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, 2>), grid, block, 0, st, xp, (const uint8_t *)w, yp, mc, N, K);
-            else
-                hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, 4>), grid, block, 0, st, xp, (const uint8_t *)w, yp, mc, N, K);
+            if (mc == 1) launch_mfma<QT, AT, 1, 8, 2>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
+            else if (mc == 2) launch_mfma<QT, AT, 1, 8, 4>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
+            else if (mc <= 4) launch_mfma<QT, AT, 1, 8, 8>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
+            else if (mc <= 8) launch_mfma<QT, AT, 2, 4, 8>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
+            else launch_mfma<QT, AT, 4, 2, 8>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
         }
         return 0;
     }
