@@ -4,9 +4,12 @@
 A "step" is one pass of the hot path over one batch of synthetic input: the
 Llama-2-7B decode linear sweep of BASELINE.json configs[1] - 32 layers x
 (q, k, v, o [4096x4096], gate, up [11008x4096], down [4096x11008]) in sym_int4,
-fp16 activations at M = 1, every linear a separate dependent launch.  The 224
-launches of a sweep are captured once in a HIP graph and replayed, so that
-Python launch cost is not billed as bandwidth.  Weights (3.64 GB) are resident
+fp16 activations at M = 1, every linear a separate launch.  The 224 launches of
+a sweep are captured once in a HIP graph and replayed, so that Python launch
+cost is not billed as bandwidth.  The seven linears of a layer are chained on
+one stream; --parallel-branches instead captures q|k|v and gate|up as parallel
+graph branches (measured slower on MI355X: cross-queue dependencies cost more
+than the overlap gains).  Weights (3.64 GB) are resident
 in HBM before the timed region and exceed the 256 MB Infinity Cache, so every
 sweep streams them from HBM.
 
@@ -43,6 +46,10 @@ def main():
     ap.add_argument("--m", type=int, default=1, help="rows of x (decode batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the M=4/8 and single-shape figures")
+    ap.add_argument("--parallel-branches", action="store_true",
+                    help="capture q|k|v and gate|up as parallel graph branches instead of one chain")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="run only the serialized [11008 x 4096] GEMV loop the roofline object is measured on")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no sharding, no collectives); --gpus must be 1",
@@ -82,15 +89,37 @@ def main():
     def make_io(m):
         xs = {k: torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32).half()
               for k in (4096, 11008)}
-        ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for n in (4096, 11008)}
+        ys = {name: torch.empty((m, n), dtype=torch.float16, device=dev) for name, n, _ in LLAMA2_7B}
         return xs, ys
 
+    side = [torch.cuda.Stream(), torch.cuda.Stream()]
+
     def sweep(m, xs, ys):
-        st = stream()
+        def run(mod):
+            name, n, k, blob = mod
+            ggml.lowbit_forward(xs[k].data_ptr(), blob.data_ptr(), ys[name].data_ptr(), SYM_INT4,
+                                ggml.LAYOUT_TILED, ggml.DT_F16, m, n, k, stream())
+
+        def branches(group):
+            # first member on the current stream, the others on side streams, then join
+            cur = torch.cuda.current_stream()
+            for s_, mod in zip(side, group[1:]):
+                s_.wait_stream(cur)
+                with torch.cuda.stream(s_):
+                    run(mod)
+            run(group[0])
+            for s_, _ in zip(side, group[1:]):
+                cur.wait_stream(s_)
+
         for mods in layers:
-            for _, n, k, blob in mods:
-                ggml.lowbit_forward(xs[k].data_ptr(), blob.data_ptr(), ys[n].data_ptr(), SYM_INT4,
-                                    ggml.LAYOUT_TILED, ggml.DT_F16, m, n, k, st)
+            if not args.parallel_branches:
+                for mod in mods:
+                    run(mod)
+            else:
+                branches(mods[0:3])      # q, k, v
+                run(mods[3])             # o
+                branches(mods[4:6])      # gate, up
+                run(mods[6])             # down
 
     def capture(fn):
         side = torch.cuda.Stream()
@@ -125,6 +154,29 @@ def main():
         return w_bytes + io
 
     xs, ys = make_io(args.m)
+
+    # ---- roofline leg: the metric's single shape (N=11008, K=4096) as a serialized chain of
+    # launches cycling over the 64 distinct gate/up weights (1.6 GB, far beyond the Infinity Cache)
+    gu = [b for mods in layers for (name, n, k, b) in mods if name in ("gate", "up")]
+
+    def headline():
+        st = stream()
+        for b in gu:
+            ggml.lowbit_forward(xs[4096].data_ptr(), b.data_ptr(), ys["gate"].data_ptr(), SYM_INT4,
+                                ggml.LAYOUT_TILED, ggml.DT_F16, args.m, 11008, 4096, st)
+    g3 = capture(headline)
+    ms3 = time_graph(g3, max(5, args.steps), max(3, args.warmup))
+    hb = blob_bytes(11008, 4096) + args.m * 4096 * 2 + args.m * 11008 * 2
+    us = ms3 * 1e3 / len(gu)
+    roofline = {"bound": "hbm", "kernel": "gemv_mfma_kernel<sym_int4,f16> on [11008 x 4096], M=%d" % args.m,
+                "achieved": round(hb / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(hb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                "bytes_per_launch": hb, "avg_launch_us": round(us, 3),
+                "how": "HIP events around graph replays of 64 chained launches over 64 distinct weights"}
+    if args.roofline_only:
+        print(json.dumps({"roofline": roofline}))
+        return
+
     g = capture(lambda: sweep(args.m, xs, ys))
     ms = time_graph(g, args.steps, args.warmup)
     total = sweep_bytes(args.m)
@@ -144,19 +196,14 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "Llama-2-7B decode linear sweep (BASELINE configs[1]): 32 layers x 7 "
-                               "linears, sym_int4, fp16 x, one launch per linear, HIP-graph replay",
+                               "linears, sym_int4, fp16 x, one launch per linear, HIP-graph replay, " +
+                               ("7 chained launches per layer" if not args.parallel_branches else
+                                "q|k|v and gate|up as parallel graph branches"),
                    "M": args.m, "launches_per_step": launches, "weight_bytes_per_step": w_bytes,
                    "algorithmic_bytes_per_step": total},
         "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
     }
-    # dominant kernel = the streaming GEMV (one symbol for all 7 shapes); a launch processes on
-    # average 1/224 of the sweep's algorithmic bytes
-    per_launch = total / launches
-    avg_us = ms * 1e3 / launches
-    out["roofline"] = {"bound": "hbm", "kernel": "gemv_mfma_kernel<sym_int4,f16>",
-                       "achieved": round(per_launch / (avg_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
-                       "unit": "GB/s", "frac": round(per_launch / (avg_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                       "traffic": None, "bytes_per_launch": round(per_launch), "avg_launch_us": round(avg_us, 3)}
+    out["roofline"] = roofline
 
     if not args.no_extra:
         extra = {}
@@ -169,22 +216,6 @@ def main():
             extra[f"sweep_M{m}"] = {"ms_per_step": round(ms2, 4),
                                     "GB/s": round(sweep_bytes(m) / (ms2 * 1e-3) / 1e9, 1)}
             del g2
-        # the metric's single shape, K=4096 N=11008, cycling over the 64 distinct gate/up weights
-        # (1.6 GB, far beyond the Infinity Cache)
-        gu = [b for mods in layers for (name, n, k, b) in mods if name in ("gate", "up")]
-
-        def headline():
-            st = stream()
-            for b in gu:
-                ggml.lowbit_forward(xs[4096].data_ptr(), b.data_ptr(), ys[11008].data_ptr(), SYM_INT4,
-                                    ggml.LAYOUT_TILED, ggml.DT_F16, args.m, 11008, 4096, st)
-        g3 = capture(headline)
-        ms3 = time_graph(g3, max(5, args.steps // 2), 3)
-        hb = blob_bytes(11008, 4096) + args.m * 4096 * 2 + args.m * 11008 * 2
-        us = ms3 * 1e3 / len(gu)
-        extra["gemv_N11008_K4096"] = {"us_per_launch": round(us, 3), "GB/s": round(hb / (us * 1e-6) / 1e9, 1),
-                                      "pct_hbm_peak": round(100 * hb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 2),
-                                      "algorithmic_bytes": hb}
         # prefill: one [11008 x 4096] linear at M = 2048
         m = 2048
         xp = torch.randn((m, 4096), generator=gen, device=dev, dtype=torch.float32).half()
@@ -194,7 +225,7 @@ def main():
             st = stream()
             for b in gu[:8]:
                 ggml.lowbit_forward(xp.data_ptr(), b.data_ptr(), yp.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED,
-                                    ggml.DT_F16, m, 11008, 4096, st)
+                                    ggml.DT_F16, 2048, 11008, 4096, st)
         g4 = capture(prefill)
         ms4 = time_graph(g4, 5, 2) / 8
         flop = 2.0 * m * 11008 * 4096
@@ -237,7 +268,7 @@ def cpu_baseline(mods, m, ggml, torch):
         one_pass()
         passes += 1
         dt = time.perf_counter() - t0
-        if dt > 10.0 or passes >= 200:
+        if dt > 10.0:
             break
     return {"value": round(nbytes * passes / dt / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"1 of 32 layers (7 linears, {nbytes} algorithmic bytes) x {passes} passes, "
