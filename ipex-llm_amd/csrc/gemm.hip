@@ -1,13 +1,300 @@
-// Prefill product (large M).  Placeholder dispatch until the MFMA GEMM lands:
-// runs the streaming kernel over 16-row slices of x.
-#include "lowbit_formats.h"
+// Prefill product y[M,N] = x[M,K] * dequant(W)[N,K]^T for large M (compute-bound).
+//
+// Replaces xe_linear.forward_new at large M
+// (python/llm/src/ipex_llm/transformers/low_bit_linear.py:660-668).
+//
+// Workgroup tile: 128 rows of x (M) by 256 weight rows (N), 4 waves side by side along N,
+// so that every weight is dequantized by exactly one wave.  Per 128-column step of K:
+//   weights: each lane loads its 16/32 bytes of four tiles straight from HBM into registers -
+//            the tiled layout already is the MFMA operand layout - and turns them into scaled
+//            fp16 / bf16 values in registers (no LDS for weights);
+//   x:       the workgroup copies the 128 x 128 block of x into LDS in operand order
+//            (double buffered), and every wave reads it from there;
+//   32 v_mfma_f32_16x16x32 per 32 columns and wave, weights as the A operand (rows = n) and x
+//   as the B operand (columns = m), so a lane ends up with 4 consecutive n for one m and
+//   stores 8 contiguous bytes of y.
+// FLOP per launch: 2*M*N*K; MFMA-bound (fp16 / bf16 dense peak).
+#include "lowbit_mfma.h"
 
 namespace lowbit {
+
 int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 int waves, hipStream_t st);
 
+constexpr int GM = 128;          // rows of x per workgroup
+constexpr int GN_WAVE = 64;      // weight rows per wave
+constexpr int GN = 256;          // weight rows per workgroup (4 waves)
+constexpr int MB = GM / 16;      // 16-row blocks of x per workgroup
+constexpr int NB = GN_WAVE / 16; // 16-row blocks of W per wave
+
+// ---- raw codes of sub-block s of a tile -> 8 *scaled* weights in the activation type ------
+
+template <int QT, typename AT> struct Dequant;
+
+__device__ inline f16x2 h2(uint32_t bits16) {
+    const uint32_t p = (bits16 & 0xffffu) | (bits16 << 16);
+    return __builtin_bit_cast(f16x2, p);
+}
+
+template <> struct Dequant<QT_SYM_INT4, _Float16> {
+    __device__ static f16x8 run(const TileRegs<QT_SYM_INT4> &t, int s, const void *) {
+        const uint32_t hb = t.h[s >> 1];
+        const f16x2 d2 = h2((s & 1) ? (hb >> 16) : hb);
+        const f16x2 k1032 = {(_Float16)1032.0f, (_Float16)1032.0f};
+        const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
+        const f16x2 k72 = {(_Float16)72.0f, (_Float16)72.0f};
+        const uint32_t v = t.q0[s], v8 = v >> 8;
+        // exact q - 8 first, one rounding in the multiply by d
+        f16x2 t0 = (__builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1032) * d2;
+        f16x2 t1 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k72) * d2;
+        f16x2 t2 = (__builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, 0x64006400u)) - k1032) * d2;
+        f16x2 t3 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, 0x64006400u)), k16th, -k72) * d2;
+        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+    }
+};
+
+template <> struct Dequant<QT_ASYM_INT4, _Float16> {
+    __device__ static f16x8 run(const TileRegs<QT_ASYM_INT4> &t, int s, const void *) {
+        const f16x2 d2 = h2(t.h[s]), m2 = h2(t.h[s] >> 16);
+        const f16x2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+        const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
+        const f16x2 k64 = {(_Float16)64.0f, (_Float16)64.0f};
+        const uint32_t v = t.q0[s], v8 = v >> 8;
+        f16x2 t0 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1024, d2, m2);
+        f16x2 t1 = __builtin_elementwise_fma(
+            __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k64), d2, m2);
+        f16x2 t2 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, 0x64006400u)) - k1024, d2, m2);
+        f16x2 t3 = __builtin_elementwise_fma(
+            __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, 0x64006400u)), k16th, -k64), d2, m2);
+        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+    }
+};
+
+// 4-bit integer codes with bf16 activations: bf16 has no packed arithmetic on gfx950, so the
+// weight is formed in fp32 ((128 + q) comes for free as a bit pattern) and rounded once.
+template <int QT> struct DequantInt4Bf16 {
+    __device__ static bf16x8 run(const TileRegs<QT> &t, int s, const void *) {
+        float d, mn;
+        tile_scale<QT>(t, s, d, mn);
+        const float off = (QT == QT_SYM_INT4) ? 136.0f : 128.0f;
+        const float c = mn - off * d;
+        const uint32_t v = t.q0[s];
+        bf16x8 r;
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint32_t pr = and_or(v >> (4 * p), 0x000f000fu, 0x43004300u);   // bf16 pair 128+q
+            const float lo = __builtin_bit_cast(float, pr << 16);
+            const float hi = __builtin_bit_cast(float, pr & 0xffff0000u);
+            r[2 * p] = (__bf16)fmaf(lo, d, c);
+            r[2 * p + 1] = (__bf16)fmaf(hi, d, c);
+        }
+        return r;
+    }
+};
+template <> struct Dequant<QT_SYM_INT4, __bf16> : DequantInt4Bf16<QT_SYM_INT4> {};
+template <> struct Dequant<QT_ASYM_INT4, __bf16> : DequantInt4Bf16<QT_ASYM_INT4> {};
+
+template <> struct Dequant<QT_SYM_INT8, _Float16> {
+    __device__ static f16x8 run(const TileRegs<QT_SYM_INT8> &t, int s, const void *) {
+        const uint32_t hb = t.h[s >> 1];
+        const f16x2 d2 = h2((s & 1) ? (hb >> 16) : hb);
+        const uint32_t lo = (s < 2 ? t.q0[2 * s] : t.q1[2 * (s - 2)]) ^ 0x80808080u;
+        const uint32_t hi = (s < 2 ? t.q0[2 * s + 1] : t.q1[2 * (s - 2) + 1]) ^ 0x80808080u;
+        const f16x2 k1152 = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const uint32_t c64 = 0x64646464u;
+        f16x2 t0 = (__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, lo, 0x04010400u)) - k1152) * d2;
+        f16x2 t1 = (__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, lo, 0x04030402u)) - k1152) * d2;
+        f16x2 t2 = (__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, hi, 0x04010400u)) - k1152) * d2;
+        f16x2 t3 = (__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, hi, 0x04030402u)) - k1152) * d2;
+        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+    }
+};
+
+template <> struct Dequant<QT_SYM_INT8, __bf16> {
+    __device__ static bf16x8 run(const TileRegs<QT_SYM_INT8> &t, int s, const void *) {
+        float d, mn;
+        tile_scale<QT_SYM_INT8>(t, s, d, mn);
+        const uint32_t lo = s < 2 ? t.q0[2 * s] : t.q1[2 * (s - 2)];
+        const uint32_t hi = s < 2 ? t.q0[2 * s + 1] : t.q1[2 * (s - 2) + 1];
+        bf16x8 r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            r[i] = (__bf16)((float)(int8_t)(lo >> (8 * i)) * d);
+            r[4 + i] = (__bf16)((float)(int8_t)(hi >> (8 * i)) * d);
+        }
+        return r;
+    }
+};
+
+// fp8: exact hardware conversion to fp32, fp32 product with the block scale, one rounding
+template <typename AT> struct Dequant<QT_FP8_E4M3, AT> {
+    __device__ static typename Vec8<AT>::type run(const TileRegs<QT_FP8_E4M3> &t, int s, const void *) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        const float sc = __builtin_bit_cast(float, t.h[0]);
+        const uint32_t lo = s < 2 ? t.q0[2 * s] : t.q1[2 * (s - 2)];
+        const uint32_t hi = s < 2 ? t.q0[2 * s + 1] : t.q1[2 * (s - 2) + 1];
+        const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
+        const f32x2 e = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), f = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+        typename Vec8<AT>::type r;
+        r[0] = to_at<AT>(a[0] * sc); r[1] = to_at<AT>(a[1] * sc); r[2] = to_at<AT>(b[0] * sc); r[3] = to_at<AT>(b[1] * sc);
+        r[4] = to_at<AT>(e[0] * sc); r[5] = to_at<AT>(e[1] * sc); r[6] = to_at<AT>(f[0] * sc); r[7] = to_at<AT>(f[1] * sc);
+        return r;
+    }
+};
+
+// nf4: fp32 code book in LDS, one rounding after the scale
+template <typename AT> struct Dequant<QT_NF4, AT> {
+    __device__ static typename Vec8<AT>::type run(const TileRegs<QT_NF4> &t, int s, const void *lut_) {
+        const float *lut = (const float *)lut_;
+        const float d = h2f((s >> 1) ? (t.h[0] >> 16) : (t.h[0] & 0xffff));
+        const uint32_t v = t.q0[s];
+        typename Vec8<AT>::type r;
+        r[0] = to_at<AT>(lut[v & 0xf] * d); r[2] = to_at<AT>(lut[(v >> 4) & 0xf] * d);
+        r[4] = to_at<AT>(lut[(v >> 8) & 0xf] * d); r[6] = to_at<AT>(lut[(v >> 12) & 0xf] * d);
+        r[1] = to_at<AT>(lut[(v >> 16) & 0xf] * d); r[3] = to_at<AT>(lut[(v >> 20) & 0xf] * d);
+        r[5] = to_at<AT>(lut[(v >> 24) & 0xf] * d); r[7] = to_at<AT>(lut[v >> 28] * d);
+        return r;
+    }
+};
+
+// ------------------------------------------------------------------ kernel
+
+template <int QT, typename AT>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+                                                        AT *__restrict__ y, int M, int N, int K) {
+    using F = Fmt<QT>;
+    using V8 = typename Vec8<AT>::type;
+    // x block in operand order: [buffer][sub-step s (4)][m-block (MB)][lane (64)] x 16 bytes
+    __shared__ __attribute__((aligned(16))) uint8_t xs[2][4 * MB * 1024];
+    __shared__ float lut[16];
+    if constexpr (QT == QT_NF4) {
+        if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODEBOOK[threadIdx.x];
+    }
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, c = lane >> 4;
+    const int G = K / TILE_COLS;
+    const int m0 = blockIdx.y * GM;
+    const int n0 = blockIdx.x * GN + wave * GN_WAVE;
+    const int n_tiles = N / TILE_ROWS;
+
+    // weight tile rows of this wave (clamped: a tile row past N is computed and never stored)
+    const uint8_t *wt[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        int tr = n0 / TILE_ROWS + nb;
+        tr = tr < n_tiles ? tr : n_tiles - 1;
+        wt[nb] = w + (int64_t)tr * G * F::TILE_BYTES;
+    }
+    // the 8 chunks of x this thread copies per K step: block b = i*4 + wave -> (s = b & 3, mb = b >> 2)
+    const AT *xg[8];
+    int xl[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int b = i * 4 + wave, s = b & 3, mb = b >> 2;
+        int row = m0 + mb * 16 + r;
+        row = row < M ? row : M - 1;
+        xg[i] = x + (int64_t)row * K + s * 32 + c * 8;
+        xl[i] = (s * MB + mb) * 1024 + lane * 16;
+    }
+
+    f32x4 acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    u32x4 xr[8];
+    TileRegs<QT> tr[NB];
+#pragma unroll
+    for (int i = 0; i < 8; i++) xr[i] = *(const u32x4 *)(xg[i]);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) load_tile<QT>(wt[nb], lane, r, tr[nb]);
+#pragma unroll
+    for (int i = 0; i < 8; i++) *(u32x4 *)(xs[0] + xl[i]) = xr[i];
+    __syncthreads();
+
+    for (int kt = 0; kt < G; kt++) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < G;
+        TileRegs<QT> tn[NB];
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) xr[i] = *(const u32x4 *)(xg[i] + (int64_t)(kt + 1) * TILE_COLS);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) load_tile<QT>(wt[nb] + (int64_t)(kt + 1) * F::TILE_BYTES, lane, r, tn[nb]);
+        }
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            V8 wv[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) wv[nb] = Dequant<QT, AT>::run(tr[nb], s, lut);
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                const V8 xv = *(const V8 *)(xs[cur] + (s * MB + mb) * 1024 + lane * 16);
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++) acc[mb][nb] = mfma16(wv[nb], xv, acc[mb][nb]);
+            }
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) *(u32x4 *)(xs[cur ^ 1] + xl[i]) = xr[i];
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) tr[nb] = tn[nb];
+        }
+        __syncthreads();
+    }
+
+    // C layout: lane = 16*g + col (col = x row within the m-block), register i = weight row 4*g + i
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        const int m = m0 + mb * 16 + r;
+        if (m < M) {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                const int n = n0 + nb * 16 + c * 4;
+                if (n < N) {
+                    typedef AT at4 __attribute__((ext_vector_type(4)));
+                    at4 o;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][i]);
+                    *(at4 *)(y + (int64_t)m * N + n) = o;
+                }
+            }
+        }
+    }
+}
+
+template <int QT, typename AT>
+static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, int K, hipStream_t st) {
+    dim3 grid((N + GN - 1) / GN, (M + GM - 1) / GM);
+    hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M,
+                       N, K);
+    return 0;
+}
+
+template <int QT>
+static int launch_gemm_q(const void *x, const void *w, void *y, int dt, int M, int N, int K, hipStream_t st) {
+    if (dt == DT_F16) return launch_gemm_t<QT, _Float16>(x, w, y, M, N, K, st);
+    if (dt == DT_BF16) return launch_gemm_t<QT, __bf16>(x, w, y, M, N, K, st);
+    return -4;
+}
+
 int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 hipStream_t st) {
-    return launch_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, st);
+    if (M == 0 || N == 0) return 0;
+    // the MFMA GEMM reads the tiled layout and stores 8-byte groups of y (N % 4 == 0 is implied
+    // by N % 16 == 0); anything else goes through the streaming kernel in 16-row slices
+    if (layout != LAYOUT_TILED || (N % TILE_ROWS) || (K % TILE_COLS) || (((uintptr_t)y) & 7))
+        return launch_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, st);
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_gemm_q<QT_SYM_INT4>(x, w, y, act_dtype, M, N, K, st);
+    case QT_ASYM_INT4: return launch_gemm_q<QT_ASYM_INT4>(x, w, y, act_dtype, M, N, K, st);
+    case QT_SYM_INT8: return launch_gemm_q<QT_SYM_INT8>(x, w, y, act_dtype, M, N, K, st);
+    case QT_NF4: return launch_gemm_q<QT_NF4>(x, w, y, act_dtype, M, N, K, st);
+    case QT_FP8_E4M3: return launch_gemm_q<QT_FP8_E4M3>(x, w, y, act_dtype, M, N, K, st);
+    default: return -2;
+    }
 }
+
 }  // namespace lowbit

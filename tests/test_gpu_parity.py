@@ -164,3 +164,41 @@ def test_headline_shape_sym_int4_m1():
     y_ref = orc.mul_mat_q(blob_np, xf, (n, k), Q4_0)
     assert np.abs(y - y_exact).max() <= 1.5e-3 * np.abs(y_exact).max()
     assert np.abs(y - y_ref).max() <= 1e-2 * np.abs(y_ref).max()
+
+
+# ------------------------------------------------------------------ MFMA GEMM (prefill)
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(17, 64, 128), (128, 256, 512), (200, 272, 384), (513, 512, 1024)])
+def test_gemm_against_oracle(qtype, dtype, m, n, k):
+    w = weights(5000 + qtype + m, (n, k))
+    x = acts(5100 + m, m, k, dtype)
+    blob_np = orc.quantize(w, qtype)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n, fn="gemm")
+    xf = x.float().numpy()
+    y_exact = orc.mul_mat_exact(blob_np, xf, (n, k), qtype)
+    assert np.isfinite(y).all()
+    tol = 2e-3 if dtype == torch.float16 else 8e-3
+    assert np.abs(y - y_exact).max() <= tol * np.abs(y_exact).max()
+    if m <= 128:
+        y_ref = orc.mul_mat_q(blob_np, xf, (n, k), qtype)
+        assert np.abs(y - y_ref).max() <= 1e-2 * np.abs(y_ref).max()
+
+
+def test_gemm_prefill_shape_sym_and_asym_int4():
+    # one Llama-2-7B linear at prefill length: [4096 x 4096], M = 512, fp16 (BASELINE configs[2])
+    n = k = 4096
+    m = 512
+    x = acts(5201, m, k, torch.float16)
+    for qtype in (Q4_0, Q4_1):
+        w = weights(5200 + qtype, (n, k))
+        blob_np = orc.quantize(w, qtype)
+        blob = dev_quantize(w, qtype, TILED)
+        y = dev_matmul(x, blob, qtype, TILED, n)
+        # oracle on a slice of the outputs keeps the CPU side to seconds
+        rows = np.arange(0, m, 37)
+        wd = orc.dequantize(blob_np, qtype, (n, k)).astype(np.float64)
+        y_exact = x.float().numpy()[rows].astype(np.float64) @ wd.T
+        assert np.abs(y[rows] - y_exact).max() <= 2e-3 * np.abs(y_exact).max()
