@@ -1,0 +1,176 @@
+"""Host logic of the drop-in Python layer and the C ABI surface; no GPU needed."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+from torch import nn
+
+import ipex_llm.ggml.model.llama.llama_cpp as ggml
+from ipex_llm.ggml.quantize import ggml_tensor_qtype
+from ipex_llm.transformers.convert import _replace_with_low_bit_linear, ggml_convert_low_bit
+from ipex_llm.transformers.low_bit_linear import (FP16Linear, FP4Params, LowBitLinear, ggml_convert_qtype,
+                                                  reshape_lm_head_input, use_batch_forward)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+Q = ggml_tensor_qtype
+
+
+def test_qtype_table_matches_reference_integers():
+    # python/llm/src/ipex_llm/ggml/quantize.py:28-57
+    assert (Q["sym_int4"], Q["asym_int4"], Q["sym_int8"], Q["nf4"], Q["fp8_e4m3"]) == (2, 3, 8, 10, 15)
+    assert (Q["fp16"], Q["bf16"], Q["fp8"], Q["fp8_e5m2"], Q["woq_int4"]) == (12, 20, 19, 19, 34)
+
+
+def test_library_exports_every_declared_symbol():
+    hdr = open(os.path.join(ROOT, "include", "lowbit_abi.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    names = re.findall(r"\b((?:lowbit|ggml|llama)_\w+)\s*\(", hdr)
+    assert len(set(names)) >= 18
+    lib = ctypes.CDLL(os.path.join(ROOT, "ipex-llm_amd", "ipex_llm", "libs", "liblowbit_hip.so"))
+    for n in set(names):
+        assert hasattr(lib, n), n
+    assert lib.lowbit_abi_version() == 1
+
+
+def test_block_geometry_through_the_abi():
+    got = [(ggml.ggml_qk_size(q), ggml.ggml_type_size(q)) for q in (2, 3, 8, 10, 15)]
+    assert got == [(32, 18), (32, 20), (32, 34), (64, 34), (128, 132)]
+    assert ggml.ggml_qk_size(Q["q4_k"]) == 0
+    assert ggml.lowbit_blob_bytes(2, 4096 * 4096) == 9437184
+    assert ggml.lowbit_blob_bytes(2, 11008 * 4096) == 25362432
+    assert ggml.lowbit_tileable(2, 4096, 11008) and not ggml.lowbit_tileable(2, 4096, 4544)
+    assert not ggml.lowbit_tileable(2, 100, 4096)
+
+
+def test_abi_rejects_bad_arguments_without_touching_the_gpu():
+    lib = ggml._lib
+    assert lib.lowbit_quantize(None, None, 99, 16, 128, 0, None) == -2
+    assert b"qtype" in lib.lowbit_last_error()
+    assert lib.lowbit_quantize(None, None, 2, 16, 100, 0, None) == -5
+    assert lib.lowbit_quantize(None, None, 2, 8, 128, 1, None) == -5       # not tileable
+    assert lib.lowbit_quantize(None, None, 2, 16, 128, 0, None) == -1      # null pointers
+    assert lib.lowbit_gemv(None, None, None, 2, 0, 2, 1, 16, 128, 0, None) == -4   # fp32 activations
+    assert lib.lowbit_relayout(ctypes.c_void_p(4096), ctypes.c_void_p(4096 + 16), 2, 16, 128, 0, None) == -1
+    assert b"overlap" in lib.lowbit_last_error()
+    assert lib.lowbit_quantize(None, None, 2, 0, 128, 0, None) == 0        # empty tensor is fine
+    with pytest.raises(RuntimeError):
+        ggml.lowbit_quantize(None, None, 99, 16, 128, 0, None)
+
+
+def test_unsupported_quantizers_raise():
+    for f in (ggml.ggml_quantize_tensor_rtn, ggml.ggml_quantize_tensor_with_weights):
+        with pytest.raises(RuntimeError):
+            f()
+
+
+@pytest.mark.parametrize("name,per_block", [("sym_int4", (32, 18)), ("asym_int4", (32, 20)),
+                                            ("sym_int8", (32, 34)), ("fp8_e4m3", (128, 132))])
+def test_convert_qtype_shape_only(name, per_block):
+    w = torch.empty(8, 256, dtype=torch.float32, device="meta")
+    out = ggml_convert_qtype(w, Q[name], device="meta")
+    assert out.dtype == torch.uint8 and out.dim() == 1
+    assert out.numel() == 8 * 256 // per_block[0] * per_block[1]
+    out2 = ggml_convert_qtype(torch.zeros(8, 256), Q[name], device="cpu", convert_shape_only=True)
+    assert out2.shape == out.shape and out2.device.type == "cpu"
+
+
+def test_convert_qtype_nf4_is_declared_bfloat16():
+    # low_bit_linear.py:132-138 of the reference: half as many bf16 elements as bytes
+    out = ggml_convert_qtype(torch.empty(4, 128, device="meta"), Q["nf4"], device="meta")
+    assert out.dtype == torch.bfloat16 and out.numel() == 4 * 128 // 64 * 34 // 2
+
+
+def test_convert_qtype_input_checks():
+    with pytest.raises(RuntimeError, match="float32"):
+        ggml_convert_qtype(torch.zeros(2, 64, dtype=torch.float16), Q["sym_int4"], device="meta")
+    with pytest.raises(RuntimeError, match="multiple of 32"):
+        ggml_convert_qtype(torch.zeros(2, 48), Q["sym_int4"], device="meta")
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        ggml_convert_qtype(torch.zeros(2, 64), Q["fp8_e4m3"], device="meta")
+    with pytest.raises(RuntimeError, match="no MI355X kernel"):
+        ggml_convert_qtype(torch.zeros(2, 256), Q["q4_k"], device="meta")
+    with pytest.raises(RuntimeError, match="scale_search"):
+        ggml_convert_qtype(torch.zeros(2, 256), Q["fp8_e4m3"], device="meta", enable_scale_search=True)
+
+
+def test_fp4params_meta_quantize_keeps_shape_bookkeeping():
+    p = FP4Params(torch.empty(16, 128, device="meta"), qtype=Q["sym_int4"])
+    q = p.to("meta")
+    assert q.quantized and tuple(q._shape) == (16, 128) and q.qtype == 2
+    assert q.data.numel() == 16 * 128 // 32 * 18 and q.get_shape() == q._shape
+    assert not q.requires_grad
+
+
+class _Toy(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.embed = nn.Embedding(10, 128)
+        self.block = nn.Sequential(nn.Linear(128, 256, bias=True), nn.ReLU(), nn.Linear(256, 128, bias=False))
+        self.odd = nn.Linear(100, 64)          # in_features % 64 != 0 -> kept
+        self.keep_me = nn.Linear(128, 128)
+        self.lm_head = nn.Linear(128, 10, bias=False)
+
+
+def test_replace_with_low_bit_linear_rules():
+    with torch.device("meta"):
+        m = _Toy()
+    m.eval()
+    m, replaced = _replace_with_low_bit_linear(m, Q["sym_int4"], modules_to_not_convert=["keep_me"],
+                                               convert_shape_only=True)
+    assert replaced
+    assert isinstance(m.block[0], LowBitLinear) and isinstance(m.block[2], LowBitLinear)
+    assert type(m.odd) is nn.Linear and type(m.keep_me) is nn.Linear and type(m.embed) is nn.Embedding
+    assert m.block[0].bias is not None and m.block[2].bias is None
+    assert m.block[0].weight.quantized and tuple(m.block[0].weight._shape) == (256, 128)
+    assert m.block[0].weight.data.numel() == 256 * 128 // 32 * 18
+    assert not m.block[0].training and not m.block[0].weight.requires_grad
+    assert m.lm_head.optimize_lm_head and not m.block[0].optimize_lm_head
+    assert (m.block[0].in_len, m.block[0].out_len, m.block[0].weight_shape) == (128, 256, (256, 128))
+    # converting twice leaves LowBitLinear layers alone
+    m, replaced = _replace_with_low_bit_linear(m, Q["sym_int4"], modules_to_not_convert=["keep_me"],
+                                               convert_shape_only=True)
+    assert isinstance(m.block[0], LowBitLinear)
+
+
+def test_convert_low_bit_fp16_and_warning():
+    m = nn.Sequential(nn.Linear(64, 64))
+    m = ggml_convert_low_bit(m, Q["fp16"])
+    assert isinstance(m[0], FP16Linear) and m[0].weight.dtype == torch.float16
+    with pytest.warns(UserWarning, match="No linear modules"):
+        ggml_convert_low_bit(nn.Sequential(nn.ReLU()), Q["sym_int4"])
+
+
+def test_optimize_model_argument_checks():
+    from ipex_llm import optimize_model
+    with pytest.raises(RuntimeError, match="Unknown load_in_low_bit"):
+        optimize_model(nn.Linear(64, 64), low_bit="int3")
+    with pytest.raises(RuntimeError, match="torch.nn.Module"):
+        optimize_model(object())
+
+
+def test_lm_head_input_keeps_last_position_of_a_prefill():
+    x = torch.arange(2 * 12 * 4, dtype=torch.float32).reshape(2, 12, 4)
+    y = reshape_lm_head_input(x)
+    assert y.shape == (2, 1, 4) and torch.equal(y[:, 0], x[:, -1])
+    assert reshape_lm_head_input(x[:, :10]).shape == (2, 10, 4)
+
+
+def test_forward_of_an_empty_activation():
+    layer = LowBitLinear(128, 64, Q["sym_int4"], bias=False)
+    y = layer(torch.empty(1, 0, 128, dtype=torch.float16))
+    assert y.shape == (1, 0, 64) and y.dtype == torch.float16
+
+
+def test_use_batch_forward_window():
+    x = torch.zeros(4, 256, dtype=torch.half)
+    assert use_batch_forward(x, 2, 64) and not use_batch_forward(x[:1], 2, 64)
+    assert not use_batch_forward(torch.zeros(32, 256, dtype=torch.half), 2, 64)
+    assert not use_batch_forward(torch.zeros(4, 192, dtype=torch.half), 2, 64)
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU failure mode")
+def test_real_quantization_without_a_gpu_fails_loudly():
+    with pytest.raises(RuntimeError, match="MI355X|failed"):
+        ggml_convert_qtype(torch.zeros(2, 64), Q["sym_int4"], device="cpu")

@@ -1,0 +1,194 @@
+"""The drop-in Python layer on a real MI355X: LowBitLinear / FP4Params / optimize_model /
+from_pretrained, compared with the CPU oracle and with dense layers holding the dequantized
+weights (the A/B style of the reference's own GPU tests, test/inference_gpu/*)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+import lowbit_oracle as orc
+import ipex_llm.ggml.model.llama.llama_cpp as ggml
+from ipex_llm.ggml.quantize import ggml_tensor_qtype as Q
+from ipex_llm.transformers.low_bit_linear import (FP4Params, LowBitLinear, dequant, ggml_convert_fp32,
+                                                  ggml_convert_qtype, ggml_matmul_src1_x_src0_t)
+from gpu_util import ALL, NAMES, weights
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(w, qtype, bias=None, **kw):
+    n, k = w.shape
+    layer = LowBitLinear(k, n, qtype, bias=bias is not None, **kw)
+    layer.weight = FP4Params(torch.from_numpy(w), qtype=qtype)
+    if bias is not None:
+        layer.bias.data = torch.from_numpy(bias)
+    return layer.eval()
+
+
+@pytest.mark.parametrize("qtype", ALL)
+def test_fp4params_device_round_trip_keeps_the_ggml_bytes(qtype):
+    w = weights(7000 + qtype, (64, 256))
+    p = FP4Params(torch.from_numpy(w), qtype=qtype)
+    g = p.to("cuda")
+    assert g.quantized and g.device.type == "cuda" and tuple(g._shape) == (64, 256)
+    c = g.to("cpu")
+    blob = c.data.view(torch.uint8).numpy()
+    assert np.array_equal(blob, orc.quantize(w, qtype))
+    # quantizing on the host path (staged through the GPU) gives the same blob
+    h = FP4Params(torch.from_numpy(w), qtype=qtype).to("cpu")
+    assert h.quantized and np.array_equal(h.data.view(torch.uint8).numpy(), blob)
+    # and a quantized CPU blob moved to the GPU equals the directly quantized one
+    assert torch.equal(h.to("cuda").data.view(torch.uint8), g.data.view(torch.uint8))
+
+
+def test_convert_qtype_blob_dtypes_and_dequant_entry_points():
+    w = weights(7100, (32, 256))
+    for qtype in ALL:
+        blob = ggml_convert_qtype(torch.from_numpy(w), qtype, device="cpu")
+        assert blob.dtype == (torch.bfloat16 if qtype == Q["nf4"] else torch.uint8)
+        want = orc.dequantize(orc.quantize(w, qtype), qtype, w.shape)
+        got = ggml_convert_fp32(blob.view(torch.uint8), w.shape, w.size, qtype)
+        assert np.array_equal(got.numpy(), want)
+        dev = FP4Params(torch.from_numpy(w), qtype=qtype).to("cuda")
+        flat = dequant(torch.empty(0, dtype=torch.float32, device="cuda"), dev.data, qtype, shape=w.shape)
+        assert np.array_equal(flat.reshape(w.shape).cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_lowbitlinear_forward_matches_dense_layer_of_dequantized_weights(qtype, dtype):
+    n, k = 96, 256
+    w = weights(7200 + qtype, (n, k))
+    bias = (np.random.default_rng(1).standard_normal(n) * 0.1).astype(np.float32)
+    layer = _layer(w, qtype, bias).to("cuda")
+    wd = torch.from_numpy(orc.dequantize(orc.quantize(w, qtype), qtype, w.shape))
+    dense = nn.Linear(k, n)
+    dense.weight.data, dense.bias.data = wd, torch.from_numpy(bias)
+    torch.manual_seed(3)
+    for shape in [(1, 1, k), (2, 5, k), (3, k), (2, 40, k)]:
+        x = torch.randn(shape).to(dtype)
+        y = layer(x.cuda())
+        assert y.dtype == dtype and y.shape == shape[:-1] + (n,) and y.device.type == "cuda"
+        ref = dense(x.float())
+        tol = 3e-3 if dtype != torch.bfloat16 else 1.2e-2
+        assert (y.float().cpu() - ref).abs().max() <= tol * ref.abs().max()
+
+
+def test_lm_head_slice_act_order_and_no_bias():
+    n, k = 64, 128
+    w = weights(7300, (n, k))
+    layer = _layer(w, Q["sym_int4"], optimize_lm_head=True, act_order=True).to("cuda")
+    perm = torch.randperm(k)
+    layer.g_idx_map = perm.cuda()
+    wd = torch.from_numpy(orc.dequantize(orc.quantize(w, 2), 2, w.shape))
+    x = torch.randn(2, 12, k).half()
+    y = layer(x.cuda()).float().cpu()
+    assert y.shape == (2, 1, n)                       # a prefill keeps its last position only
+    ref = x[:, -1:, :].float()[..., perm] @ wd.T
+    assert (y - ref).abs().max() <= 3e-3 * ref.abs().max()
+
+
+def test_cpu_resident_weight_uses_the_host_pointer_matmul():
+    n, k = 48, 256
+    w = weights(7400, (n, k))
+    layer = _layer(w, Q["sym_int4"])
+    layer.weight = layer.weight.to("cpu")             # quantized, still on the host
+    x = torch.randn(3, k)
+    y = layer(x)
+    assert y.device.type == "cpu" and y.dtype == torch.float32
+    blob = orc.quantize(w, 2)
+    ref = orc.mul_mat_q(blob, x.numpy(), (n, k), 2)    # the reference's CPU low-bit matmul
+    assert np.abs(y.numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
+    y2 = ggml_matmul_src1_x_src0_t(layer.weight.data, x, (n, k), 2)
+    assert torch.equal(y, y2)
+    with pytest.raises(RuntimeError, match="not supported on CPU"):
+        l2 = _layer(w, Q["nf4"])
+        l2.weight = l2.weight.to("cpu")
+        l2(x)
+
+
+def test_host_pointer_abi_quantize_dequantize():
+    w = weights(7500, (16, 384))
+    for qtype in ALL:
+        src = np.ascontiguousarray(w)
+        dst = np.zeros(ggml.lowbit_blob_bytes(qtype, w.size), dtype=np.uint8)
+        hist = (ctypes.c_int64 * 16)()
+        n = ggml.ggml_quantize_tensor(src.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                      ctypes.c_void_p(dst.ctypes.data), qtype, w.size, w.shape[1], hist, False)
+        assert n == dst.size and np.array_equal(dst, orc.quantize(w, qtype))
+        out = np.zeros(w.size, dtype=np.float32)
+        ggml.ggml_dequantize(ctypes.c_void_p(dst.ctypes.data), ctypes.c_void_p(out.ctypes.data), w.size, qtype)
+        assert np.array_equal(out.reshape(w.shape), orc.dequantize(dst, qtype, w.shape))
+    with pytest.raises(RuntimeError, match="scale_search"):
+        ggml.ggml_quantize_tensor(src.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                  ctypes.c_void_p(dst.ctypes.data), 2, w.size, w.shape[1], hist, True)
+
+
+class _Mlp(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.up = nn.Linear(128, 256)
+        self.down = nn.Linear(256, 128, bias=False)
+        self.skip = nn.Linear(128, 128)
+
+    def forward(self, x):
+        return self.skip(self.down(torch.relu(self.up(x))))
+
+
+@pytest.mark.parametrize("low_bit", ["sym_int4", "asym_int4", "sym_int8", "nf4", "fp8_e4m3"])
+def test_optimize_model_save_and_load_low_bit(low_bit, tmp_path):
+    from ipex_llm import optimize_model
+    from ipex_llm.optimize import load_low_bit
+    torch.manual_seed(11)
+    ref = _Mlp().eval()
+    model = _Mlp().eval()
+    model.load_state_dict(ref.state_dict())
+    model = optimize_model(model, low_bit=low_bit, modules_to_not_convert=["skip"])
+    assert isinstance(model.up, LowBitLinear) and type(model.skip) is nn.Linear
+    assert model._bigdl_config["bigdl_transformers_low_bit"] == low_bit
+    x = torch.randn(4, 128)
+    model = model.to("cuda")
+    y = model(x.cuda()).cpu()
+    want = ref(x)
+    rel = (y - want).abs().max() / want.abs().max()
+    assert rel < (0.15 if "4" in low_bit else 0.05)          # quantization noise, not kernel error
+    model.save_low_bit(str(tmp_path))
+    fresh = load_low_bit(_Mlp().eval(), str(tmp_path))
+    assert isinstance(fresh.up, LowBitLinear) and fresh.up.weight.quantized
+    blob_saved = fresh.up.weight.data.view(torch.uint8).numpy()
+    assert np.array_equal(blob_saved, orc.quantize(ref.up.weight.detach().numpy(), Q[low_bit]))
+    y2 = fresh.to("cuda")(x.cuda()).cpu()
+    assert torch.equal(y, y2)
+
+
+def test_from_pretrained_tiny_llama_and_low_bit_round_trip(tmp_path):
+    transformers = pytest.importorskip("transformers")
+    from ipex_llm.transformers import AutoModelForCausalLM
+    cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=4, vocab_size=320,
+                                   max_position_embeddings=64)
+    torch.manual_seed(5)
+    hf = transformers.LlamaForCausalLM(cfg).eval()
+    src = tmp_path / "fp"
+    hf.save_pretrained(str(src))
+    model = AutoModelForCausalLM.from_pretrained(str(src), load_in_low_bit="sym_int4",
+                                                 modules_to_not_convert=["lm_head"])
+    assert model.config.bigdl_transformers_low_bit == "sym_int4"
+    lin = model.model.layers[0].mlp.gate_proj
+    assert isinstance(lin, LowBitLinear) and lin.weight.quantized
+    assert type(model.lm_head) is nn.Linear
+    ids = torch.randint(0, 320, (1, 9))
+    with torch.no_grad():
+        want = hf(ids).logits
+        got = model.to("cuda")(ids.cuda()).logits.float().cpu()
+    assert (got - want).abs().mean() / want.abs().mean() < 0.2
+    out = tmp_path / "lowbit"
+    model.save_low_bit(str(out))
+    with pytest.raises(RuntimeError, match="load_low_bit"):
+        AutoModelForCausalLM.from_pretrained(str(out), load_in_4bit=True)
+    again = AutoModelForCausalLM.load_low_bit(str(out))
+    with torch.no_grad():
+        got2 = again.to("cuda")(ids.cuda()).logits.float().cpu()
+    assert torch.equal(got, got2)
