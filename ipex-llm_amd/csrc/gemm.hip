@@ -114,14 +114,20 @@ template <> struct Dequant<QT_SYM_INT8, __bf16> {
     __device__ static bf16x8 run(const TileRegs<QT_SYM_INT8> &t, int s, const void *) {
         float d, mn;
         tile_scale<QT_SYM_INT8>(t, s, d, mn);
-        const uint32_t lo = s < 2 ? t.q0[2 * s] : t.q1[2 * (s - 2)];
-        const uint32_t hi = s < 2 ? t.q0[2 * s + 1] : t.q1[2 * (s - 2) + 1];
+        // byte ^ 0x80 = q + 128 as an unsigned byte, which v_cvt_f32_ubyteN converts exactly;
+        // (u - 128) * d is one fma in fp32, rounded once to bf16
+        const uint32_t lo = (s < 2 ? t.q0[2 * s] : t.q1[2 * (s - 2)]) ^ 0x80808080u;
+        const uint32_t hi = (s < 2 ? t.q0[2 * s + 1] : t.q1[2 * (s - 2) + 1]) ^ 0x80808080u;
+        const float c = -128.0f * d;
         bf16x8 r;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            r[i] = (__bf16)((float)(int8_t)(lo >> (8 * i)) * d);
-            r[4 + i] = (__bf16)((float)(int8_t)(hi >> (8 * i)) * d);
-        }
+        r[0] = (__bf16)fmaf((float)(lo & 0xff), d, c);
+        r[1] = (__bf16)fmaf((float)((lo >> 8) & 0xff), d, c);
+        r[2] = (__bf16)fmaf((float)((lo >> 16) & 0xff), d, c);
+        r[3] = (__bf16)fmaf((float)(lo >> 24), d, c);
+        r[4] = (__bf16)fmaf((float)(hi & 0xff), d, c);
+        r[5] = (__bf16)fmaf((float)((hi >> 8) & 0xff), d, c);
+        r[6] = (__bf16)fmaf((float)((hi >> 16) & 0xff), d, c);
+        r[7] = (__bf16)fmaf((float)(hi >> 24), d, c);
         return r;
     }
 };
@@ -159,44 +165,83 @@ template <typename AT> struct Dequant<QT_NF4, AT> {
 
 // ------------------------------------------------------------------ kernel
 
+// MFMA with the accumulator pinned to accumulation registers, in place.  Written as inline
+// assembly because the compiler otherwise lets the 128 accumulators migrate between register
+// ranges across the unrolled K steps and copies all of them back every iteration.
+__device__ inline void mfma_acc(f32x4 &c, f16x8 a, f16x8 b) {
+    asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ inline void mfma_acc(f32x4 &c, bf16x8 a, bf16x8 b) {
+    asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
 template <int QT, typename AT>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
-                                                        AT *__restrict__ y, int M, int N, int K) {
+                                                        AT *__restrict__ y, int M, int N, int K, int xcd_m) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
-    // x block in operand order: [buffer][sub-step s (4)][m-block (MB)][lane (64)] x 16 bytes
-    __shared__ __attribute__((aligned(16))) uint8_t xs[2][4 * MB * 1024];
+    // x block in operand order: [sub-step s (4)][m-block (MB)][lane (64)] x 16 bytes, two buffers
+    __shared__ __attribute__((aligned(16))) uint8_t xs0[4 * MB * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t xs1[4 * MB * 1024];
     __shared__ float lut[16];
     if constexpr (QT == QT_NF4) {
         if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODEBOOK[threadIdx.x];
     }
 
+
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, c = lane >> 4;
     const int G = K / TILE_COLS;
-    const int m0 = blockIdx.y * GM;
-    const int n0 = blockIdx.x * GN + wave * GN_WAVE;
     const int n_tiles = N / TILE_ROWS;
+
+    // Workgroups are handed to the 8 XCDs round-robin (id % 8) and each XCD has its own L2.  The
+    // output tiles are therefore dealt out so that one XCD owns a block of xm_band row-tiles by
+    // xn_band column-tiles: its L2 then only has to hold that band of x (re-read by every
+    // column-tile) and sees each weight tile from all its row-tiles at about the same time.
+    const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int band_m = (tiles_m + xcd_m - 1) / xcd_m;            // row-tiles per XCD block
+    const int xcd_n = 8 / xcd_m;
+    const int band_n = (tiles_n + xcd_n - 1) / xcd_n;            // column-tiles per XCD block
+    const int tile_m = (xcd % xcd_m) * band_m + slot % band_m;
+    const int tile_n = (xcd / xcd_m) * band_n + slot / band_m;
+    if (slot >= band_m * band_n || tile_m >= tiles_m || tile_n >= tiles_n) return;   // whole workgroup leaves
+    const int m0 = tile_m * GM;
+    const int n0 = tile_n * GN + wave * GN_WAVE;
 
     // weight tile rows of this wave (clamped: a tile row past N is computed and never stored)
     const uint8_t *wt[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
-        int tr = n0 / TILE_ROWS + nb;
-        tr = tr < n_tiles ? tr : n_tiles - 1;
-        wt[nb] = w + (int64_t)tr * G * F::TILE_BYTES;
+        int trow = n0 / TILE_ROWS + nb;
+        trow = trow < n_tiles ? trow : n_tiles - 1;
+        wt[nb] = w + (int64_t)trow * G * F::TILE_BYTES;
     }
-    // the 8 chunks of x this thread copies per K step: block b = i*4 + wave -> (s = b & 3, mb = b >> 2)
-    const AT *xg[8];
-    int xl[8];
+    // x goes global -> registers -> LDS (operand order: chunk (s, mb) of lane l at
+    // ((s*MB + mb)*64 + l) * 16 bytes).  Wave w copies sub-step s = w of every m-block.
+    uint32_t xoff[MB];                                   // byte offset of this lane's chunk, per m-block
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int b = i * 4 + wave, s = b & 3, mb = b >> 2;
+    for (int mb = 0; mb < MB; mb++) {
         int row = m0 + mb * 16 + r;
         row = row < M ? row : M - 1;
-        xg[i] = x + (int64_t)row * K + s * 32 + c * 8;
-        xl[i] = (s * MB + mb) * 1024 + lane * 16;
+        xoff[mb] = (uint32_t)(((int64_t)row * K + wave * 32 + c * 8) * (int64_t)sizeof(AT));
     }
+    const int last = G - 1;
+    auto load_x = [&](int kt, u32x4 (&xr)[MB]) {
+        kt = kt < last ? kt : last;                      // past the end: a harmless re-read, never used
+        const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) xr[mb] = *(const u32x4 *)(xk + xoff[mb]);
+    };
+    auto store_x = [&](uint8_t *buf, const u32x4 (&xr)[MB]) {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) *(u32x4 *)(buf + (wave * MB + mb) * 1024 + lane * 16) = xr[mb];
+    };
+    auto load_w = [&](int kt, TileRegs<QT> (&t)[NB]) {
+        kt = kt < last ? kt : last;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) load_tile<QT>(wt[nb] + (int64_t)kt * F::TILE_BYTES, lane, r, t[nb]);
+    };
 
     f32x4 acc[MB][NB];
 #pragma unroll
@@ -204,47 +249,58 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) acc[mb][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    u32x4 xr[8];
-    TileRegs<QT> tr[NB];
-#pragma unroll
-    for (int i = 0; i < 8; i++) xr[i] = *(const u32x4 *)(xg[i]);
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) load_tile<QT>(wt[nb], lane, r, tr[nb]);
-#pragma unroll
-    for (int i = 0; i < 8; i++) *(u32x4 *)(xs[0] + xl[i]) = xr[i];
-    __syncthreads();
-
-    for (int kt = 0; kt < G; kt++) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < G;
-        TileRegs<QT> tn[NB];
-        if (more) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) xr[i] = *(const u32x4 *)(xg[i] + (int64_t)(kt + 1) * TILE_COLS);
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) load_tile<QT>(wt[nb] + (int64_t)(kt + 1) * F::TILE_BYTES, lane, r, tn[nb]);
-        }
+    // 4 sub-steps of 32 columns; the x operands of a sub-step are requested before its weights
+    // are dequantized, so the LDS latency hides behind that VALU work.
+    auto compute = [&](const uint8_t *cur, const TileRegs<QT> (&tr)[NB]) {
 #pragma unroll
         for (int s = 0; s < 4; s++) {
+            V8 xv[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) xv[mb] = *(const V8 *)(cur + (s * MB + mb) * 1024 + lane * 16);
             V8 wv[NB];
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) wv[nb] = Dequant<QT, AT>::run(tr[nb], s, lut);
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                const V8 xv = *(const V8 *)(xs[cur] + (s * MB + mb) * 1024 + lane * 16);
+            for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                for (int nb = 0; nb < NB; nb++) acc[mb][nb] = mfma16(wv[nb], xv, acc[mb][nb]);
-            }
+                for (int nb = 0; nb < NB; nb++) mfma_acc(acc[mb][nb], wv[nb], xv[mb]);
         }
-        if (more) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) *(u32x4 *)(xs[cur ^ 1] + xl[i]) = xr[i];
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) tr[nb] = tn[nb];
-        }
-        __syncthreads();
-    }
+    };
 
+    // Software pipeline, two K steps deep: while step kt is computed, the data of step kt+1 is
+    // already in registers (it moves to LDS at the end of step kt) and the loads of step kt+2
+    // are issued.  x rotates through two register sets, the weight tiles through three, hence
+    // the period of six.
+    u32x4 xa[MB], xb[MB];
+    TileRegs<QT> w0[NB], w1[NB], w2[NB];
+    load_x(0, xa);
+    load_w(0, w0);
+    load_x(1, xb);
+    load_w(1, w1);
+    store_x(xs0, xa);
+    __syncthreads();
+
+#define LOWBIT_GEMM_STEP(i, cur, nxt, xst, xld, wc, wl) \
+    if (kt + (i) < G) {                                 \
+        load_x(kt + (i) + 2, xld);                      \
+        load_w(kt + (i) + 2, wl);                       \
+        compute(cur, wc);                               \
+        store_x(nxt, xst);                              \
+        __syncthreads();                                \
+    }
+    for (int kt = 0; kt < G; kt += 6) {
+        LOWBIT_GEMM_STEP(0, xs0, xs1, xb, xa, w0, w2)
+        LOWBIT_GEMM_STEP(1, xs1, xs0, xa, xb, w1, w0)
+        LOWBIT_GEMM_STEP(2, xs0, xs1, xb, xa, w2, w1)
+        LOWBIT_GEMM_STEP(3, xs1, xs0, xa, xb, w0, w2)
+        LOWBIT_GEMM_STEP(4, xs0, xs1, xb, xa, w1, w0)
+        LOWBIT_GEMM_STEP(5, xs1, xs0, xa, xb, w2, w1)
+    }
+#undef LOWBIT_GEMM_STEP
+
+    // the MFMAs above are opaque to the compiler's hazard tracking: give the last results time
+    // to land before the accumulation registers are read back (an 8-pass MFMA needs 18 cycles)
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");
     // C layout: lane = 16*g + col (col = x row within the m-block), register i = weight row 4*g + i
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
@@ -267,9 +323,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
 
 template <int QT, typename AT>
 static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, int K, hipStream_t st) {
-    dim3 grid((N + GN - 1) / GN, (M + GM - 1) / GM);
+    const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
+    int xcd_m = 1;                                       // XCDs along M: power of two <= min(8, tiles_m)
+    while (xcd_m * 2 <= 8 && xcd_m * 2 <= tiles_m) xcd_m *= 2;
+    const int xcd_n = 8 / xcd_m;
+    const int band_m = (tiles_m + xcd_m - 1) / xcd_m, band_n = (tiles_n + xcd_n - 1) / xcd_n;
+    dim3 grid(8 * band_m * band_n);
     hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M,
-                       N, K);
+                       N, K, xcd_m);
     return 0;
 }
 
