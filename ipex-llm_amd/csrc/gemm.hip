@@ -29,137 +29,116 @@ constexpr int NB = GN_WAVE / 16; // 16-row blocks of W per wave
 
 // ---- raw codes of sub-block s of a tile -> 8 *scaled* weights in the activation type ------
 
+// Dequant<QT, AT>::pair(t, s, p): columns 2p, 2p+1 (p = 0..3) of the lane's 8 columns of
+// sub-block s, scaled, as one packed 32-bit register.  Pair granularity lets the main loop
+// slip a few VALU instructions between consecutive MFMAs.
 template <int QT, typename AT> struct Dequant;
 
 __device__ inline f16x2 h2(uint32_t bits16) {
     const uint32_t p = (bits16 & 0xffffu) | (bits16 << 16);
     return __builtin_bit_cast(f16x2, p);
 }
+__device__ inline uint32_t pk(f16x2 v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ inline uint32_t pk(bf16x2 v) { return __builtin_bit_cast(uint32_t, v); }
+template <typename AT> __device__ inline uint32_t pk2(float a, float b);
+template <> __device__ inline uint32_t pk2<_Float16>(float a, float b) { return pk(f16x2{(_Float16)a, (_Float16)b}); }
+template <> __device__ inline uint32_t pk2<__bf16>(float a, float b) { return pk(bf16x2{(__bf16)a, (__bf16)b}); }
 
 template <> struct Dequant<QT_SYM_INT4, _Float16> {
-    __device__ static f16x8 run(const TileRegs<QT_SYM_INT4> &t, int s, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT4> &t, int s, int p, const void *) {
         const uint32_t hb = t.h[s >> 1];
         const f16x2 d2 = h2((s & 1) ? (hb >> 16) : hb);
         const f16x2 k1032 = {(_Float16)1032.0f, (_Float16)1032.0f};
         const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
         const f16x2 k72 = {(_Float16)72.0f, (_Float16)72.0f};
-        const uint32_t v = t.q0[s], v8 = v >> 8;
-        // exact q - 8 first, one rounding in the multiply by d
-        f16x2 t0 = (__builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1032) * d2;
-        f16x2 t1 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k72) * d2;
-        f16x2 t2 = (__builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, 0x64006400u)) - k1032) * d2;
-        f16x2 t3 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, 0x64006400u)), k16th, -k72) * d2;
-        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+        const uint32_t v = (p & 2) ? (t.q0[s] >> 8) : t.q0[s];
+        // exact q - 8 first (0x6400 | q is the half 1024 + q), one rounding in the multiply by d
+        if (p & 1)
+            return pk(__builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k72) * d2);
+        return pk((__builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1032) * d2);
     }
 };
 
 template <> struct Dequant<QT_ASYM_INT4, _Float16> {
-    __device__ static f16x8 run(const TileRegs<QT_ASYM_INT4> &t, int s, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_ASYM_INT4> &t, int s, int p, const void *) {
         const f16x2 d2 = h2(t.h[s]), m2 = h2(t.h[s] >> 16);
         const f16x2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
         const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
         const f16x2 k64 = {(_Float16)64.0f, (_Float16)64.0f};
-        const uint32_t v = t.q0[s], v8 = v >> 8;
-        f16x2 t0 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1024, d2, m2);
-        f16x2 t1 = __builtin_elementwise_fma(
-            __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k64), d2, m2);
-        f16x2 t2 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, 0x64006400u)) - k1024, d2, m2);
-        f16x2 t3 = __builtin_elementwise_fma(
-            __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, 0x64006400u)), k16th, -k64), d2, m2);
-        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+        const uint32_t v = (p & 2) ? (t.q0[s] >> 8) : t.q0[s];
+        f16x2 q;
+        if (p & 1) q = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k64);
+        else q = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1024;
+        return pk(__builtin_elementwise_fma(q, d2, m2));
     }
 };
 
 // 4-bit integer codes with bf16 activations: bf16 has no packed arithmetic on gfx950, so the
 // weight is formed in fp32 ((128 + q) comes for free as a bit pattern) and rounded once.
 template <int QT> struct DequantInt4Bf16 {
-    __device__ static bf16x8 run(const TileRegs<QT> &t, int s, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT> &t, int s, int p, const void *) {
         float d, mn;
         tile_scale<QT>(t, s, d, mn);
         const float off = (QT == QT_SYM_INT4) ? 136.0f : 128.0f;
         const float c = mn - off * d;
-        const uint32_t v = t.q0[s];
-        bf16x8 r;
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-            const uint32_t pr = and_or(v >> (4 * p), 0x000f000fu, 0x43004300u);   // bf16 pair 128+q
-            const float lo = __builtin_bit_cast(float, pr << 16);
-            const float hi = __builtin_bit_cast(float, pr & 0xffff0000u);
-            r[2 * p] = (__bf16)fmaf(lo, d, c);
-            r[2 * p + 1] = (__bf16)fmaf(hi, d, c);
-        }
-        return r;
+        const uint32_t pr = and_or(t.q0[s] >> (4 * p), 0x000f000fu, 0x43004300u);   // bf16 pair 128+q
+        const float lo = __builtin_bit_cast(float, pr << 16);
+        const float hi = __builtin_bit_cast(float, pr & 0xffff0000u);
+        return pk2<__bf16>(fmaf(lo, d, c), fmaf(hi, d, c));
     }
 };
 template <> struct Dequant<QT_SYM_INT4, __bf16> : DequantInt4Bf16<QT_SYM_INT4> {};
 template <> struct Dequant<QT_ASYM_INT4, __bf16> : DequantInt4Bf16<QT_ASYM_INT4> {};
 
+__device__ inline uint32_t code_word8(const u32x4 &q0, const u32x4 &q1, int s, int p) {
+    // 8-bit codes: sub-block s holds two dwords (columns 0..3, 4..7)
+    const int w = 2 * (s & 1) + (p >> 1);
+    return s < 2 ? q0[w] : q1[w];
+}
+
 template <> struct Dequant<QT_SYM_INT8, _Float16> {
-    __device__ static f16x8 run(const TileRegs<QT_SYM_INT8> &t, int s, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT8> &t, int s, int p, const void *) {
         const uint32_t hb = t.h[s >> 1];
         const f16x2 d2 = h2((s & 1) ? (hb >> 16) : hb);
-        const uint32_t lo = (s < 2 ? t.q0[2 * s] : t.q1[2 * (s - 2)]) ^ 0x80808080u;
-        const uint32_t hi = (s < 2 ? t.q0[2 * s + 1] : t.q1[2 * (s - 2) + 1]) ^ 0x80808080u;
+        // byte ^ 0x80 = q + 128 (unsigned); 0x6400 | u is the half 1024 + u
+        const uint32_t w = code_word8(t.q0, t.q1, s, p) ^ 0x80808080u;
         const f16x2 k1152 = {(_Float16)1152.0f, (_Float16)1152.0f};
-        const uint32_t c64 = 0x64646464u;
-        f16x2 t0 = (__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, lo, 0x04010400u)) - k1152) * d2;
-        f16x2 t1 = (__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, lo, 0x04030402u)) - k1152) * d2;
-        f16x2 t2 = (__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, hi, 0x04010400u)) - k1152) * d2;
-        f16x2 t3 = (__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(c64, hi, 0x04030402u)) - k1152) * d2;
-        return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+        const uint32_t sel = (p & 1) ? 0x04030402u : 0x04010400u;
+        return pk((__builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, w, sel)) - k1152) * d2);
     }
 };
 
 template <> struct Dequant<QT_SYM_INT8, __bf16> {
-    __device__ static bf16x8 run(const TileRegs<QT_SYM_INT8> &t, int s, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT8> &t, int s, int p, const void *) {
         float d, mn;
         tile_scale<QT_SYM_INT8>(t, s, d, mn);
-        // byte ^ 0x80 = q + 128 as an unsigned byte, which v_cvt_f32_ubyteN converts exactly;
-        // (u - 128) * d is one fma in fp32, rounded once to bf16
-        const uint32_t lo = (s < 2 ? t.q0[2 * s] : t.q1[2 * (s - 2)]) ^ 0x80808080u;
-        const uint32_t hi = (s < 2 ? t.q0[2 * s + 1] : t.q1[2 * (s - 2) + 1]) ^ 0x80808080u;
+        // byte ^ 0x80 = q + 128 as an unsigned byte, converted exactly; (u - 128) * d is one fp32
+        // fma, rounded once to bf16
+        const uint32_t w = (code_word8(t.q0, t.q1, s, p) ^ 0x80808080u) >> ((p & 1) * 16);
         const float c = -128.0f * d;
-        bf16x8 r;
-        r[0] = (__bf16)fmaf((float)(lo & 0xff), d, c);
-        r[1] = (__bf16)fmaf((float)((lo >> 8) & 0xff), d, c);
-        r[2] = (__bf16)fmaf((float)((lo >> 16) & 0xff), d, c);
-        r[3] = (__bf16)fmaf((float)(lo >> 24), d, c);
-        r[4] = (__bf16)fmaf((float)(hi & 0xff), d, c);
-        r[5] = (__bf16)fmaf((float)((hi >> 8) & 0xff), d, c);
-        r[6] = (__bf16)fmaf((float)((hi >> 16) & 0xff), d, c);
-        r[7] = (__bf16)fmaf((float)(hi >> 24), d, c);
-        return r;
+        return pk2<__bf16>(fmaf((float)(w & 0xff), d, c), fmaf((float)((w >> 8) & 0xff), d, c));
     }
 };
 
 // fp8: exact hardware conversion to fp32, fp32 product with the block scale, one rounding
 template <typename AT> struct Dequant<QT_FP8_E4M3, AT> {
-    __device__ static typename Vec8<AT>::type run(const TileRegs<QT_FP8_E4M3> &t, int s, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_FP8_E4M3> &t, int s, int p, const void *) {
         typedef float f32x2 __attribute__((ext_vector_type(2)));
         const float sc = __builtin_bit_cast(float, t.h[0]);
-        const uint32_t lo = s < 2 ? t.q0[2 * s] : t.q1[2 * (s - 2)];
-        const uint32_t hi = s < 2 ? t.q0[2 * s + 1] : t.q1[2 * (s - 2) + 1];
-        const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
-        const f32x2 e = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), f = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
-        typename Vec8<AT>::type r;
-        r[0] = to_at<AT>(a[0] * sc); r[1] = to_at<AT>(a[1] * sc); r[2] = to_at<AT>(b[0] * sc); r[3] = to_at<AT>(b[1] * sc);
-        r[4] = to_at<AT>(e[0] * sc); r[5] = to_at<AT>(e[1] * sc); r[6] = to_at<AT>(f[0] * sc); r[7] = to_at<AT>(f[1] * sc);
-        return r;
+        const uint32_t w = code_word8(t.q0, t.q1, s, p);
+        const f32x2 a = (p & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8(w, true) : __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+        return pk2<AT>(a[0] * sc, a[1] * sc);
     }
 };
 
-// nf4: fp32 code book in LDS, one rounding after the scale
+// nf4: fp32 code book in LDS, one rounding after the scale.  Nibble order 0,2,4,6,1,3,5,7:
+// columns 2p and 2p+1 sit in nibbles p and p+4.
 template <typename AT> struct Dequant<QT_NF4, AT> {
-    __device__ static typename Vec8<AT>::type run(const TileRegs<QT_NF4> &t, int s, const void *lut_) {
+    __device__ static uint32_t pair(const TileRegs<QT_NF4> &t, int s, int p, const void *lut_) {
         const float *lut = (const float *)lut_;
         const float d = h2f((s >> 1) ? (t.h[0] >> 16) : (t.h[0] & 0xffff));
-        const uint32_t v = t.q0[s];
-        typename Vec8<AT>::type r;
-        r[0] = to_at<AT>(lut[v & 0xf] * d); r[2] = to_at<AT>(lut[(v >> 4) & 0xf] * d);
-        r[4] = to_at<AT>(lut[(v >> 8) & 0xf] * d); r[6] = to_at<AT>(lut[(v >> 12) & 0xf] * d);
-        r[1] = to_at<AT>(lut[(v >> 16) & 0xf] * d); r[3] = to_at<AT>(lut[(v >> 20) & 0xf] * d);
-        r[5] = to_at<AT>(lut[(v >> 24) & 0xf] * d); r[7] = to_at<AT>(lut[v >> 28] * d);
-        return r;
+        const uint32_t v = t.q0[s] >> (4 * p);
+        return pk2<AT>(lut[v & 0xf] * d, lut[(v >> 16) & 0xf] * d);
     }
 };
 
@@ -249,21 +228,38 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) acc[mb][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // 4 sub-steps of 32 columns; the x operands of a sub-step are requested before its weights
-    // are dequantized, so the LDS latency hides behind that VALU work.
+    // 4 sub-steps of 32 columns, written in the order the hardware should issue them: after the
+    // MFMAs of an m-block, the x operand of that m-block for the NEXT sub-step is requested from
+    // LDS, and after every second MFMA one register pair of the next sub-step's weights is
+    // dequantized, so that LDS latency and the VALU work run in the shadow of the MFMA pipe.
     auto compute = [&](const uint8_t *cur, const TileRegs<QT> (&tr)[NB]) {
+        V8 xv[MB];
+        u32x4 wv[NB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) xv[mb] = *(const V8 *)(cur + mb * 1024 + lane * 16);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int p = 0; p < 4; p++) wv[nb][p] = Dequant<QT, AT>::pair(tr[nb], 0, p, lut);
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            V8 xv[MB];
+            u32x4 wn[NB];
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) xv[mb] = *(const V8 *)(cur + (s * MB + mb) * 1024 + lane * 16);
-            V8 wv[NB];
+            for (int mb = 0; mb < MB; mb++) {
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) wv[nb] = Dequant<QT, AT>::run(tr[nb], s, lut);
+                for (int nb = 0; nb < NB; nb++) {
+                    mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    if (s < 3 && (nb & 1)) {
+                        const int idx = mb * (NB / 2) + nb / 2;      // 0 .. 15: (weight block, pair)
+                        wn[idx >> 2][idx & 3] = Dequant<QT, AT>::pair(tr[idx >> 2], s + 1, idx & 3, lut);
+                    }
+                }
+                if (s < 3) xv[mb] = *(const V8 *)(cur + ((s + 1) * MB + mb) * 1024 + lane * 16);
+            }
+            if (s < 3) {
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-                for (int nb = 0; nb < NB; nb++) mfma_acc(acc[mb][nb], wv[nb], xv[mb]);
+                for (int nb = 0; nb < NB; nb++) wv[nb] = wn[nb];
+            }
         }
     };
 
