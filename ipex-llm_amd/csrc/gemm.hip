@@ -10,9 +10,9 @@
 //            fp16 / bf16 values in registers (no LDS for weights);
 //   x:       the workgroup copies the 128 x 128 block of x into LDS in operand order
 //            (double buffered), and every wave reads it from there;
-//   32 v_mfma_f32_16x16x32 per 32 columns and wave, weights as the A operand (rows = n) and x
-//   as the B operand (columns = m), so a lane ends up with 4 consecutive n for one m and
-//   stores 8 contiguous bytes of y.
+//   8 v_mfma_f32_32x32x16 per 16 columns and wave, weights as the A operand (rows = n) and x
+//   as the B operand (columns = m), so a lane ends up with groups of 4 consecutive n for one m
+//   and stores 8 contiguous bytes of y at a time.
 // FLOP per launch: 2*M*N*K; MFMA-bound (fp16 / bf16 dense peak).
 #include "lowbit_mfma.h"
 
@@ -24,8 +24,6 @@ int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, in
 constexpr int GM = 128;          // rows of x per workgroup
 constexpr int GN_WAVE = 64;      // weight rows per wave
 constexpr int GN = 256;          // weight rows per workgroup (4 waves)
-constexpr int MB = GM / 16;      // 16-row blocks of x per workgroup
-constexpr int NB = GN_WAVE / 16; // 16-row blocks of W per wave
 
 // ---- raw codes of sub-block s of a tile -> 8 *scaled* weights in the activation type ------
 
@@ -144,121 +142,163 @@ template <typename AT> struct Dequant<QT_NF4, AT> {
 
 // ------------------------------------------------------------------ kernel
 
-// MFMA with the accumulator pinned to accumulation registers, in place.  Written as inline
-// assembly because the compiler otherwise lets the 128 accumulators migrate between register
-// ranges across the unrolled K steps and copies all of them back every iteration.
-__device__ inline void mfma_acc(f32x4 &c, f16x8 a, f16x8 b) {
-    asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// v_mfma_f32_32x32x16: measured on MI355X at 2.3 PFLOP/s, twice the rate of the 16x16x32 form,
+// so the GEMM is built on it.  The accumulator is pinned to accumulation registers, in place,
+// through inline assembly: left to the compiler, the 128 accumulators migrate between register
+// ranges across the unrolled K steps and get copied back every iteration.
+__device__ inline void mfma_acc(f32x16 &c, f16x8 a, f16x8 b) {
+    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
-__device__ inline void mfma_acc(f32x4 &c, bf16x8 a, bf16x8 b) {
-    asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+__device__ inline void mfma_acc(f32x16 &c, bf16x8 a, bf16x8 b) {
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
+constexpr int MB32 = GM / 32;        // 32-row blocks of x per workgroup
+constexpr int NB32 = GN_WAVE / 32;   // 32-row blocks of W per wave (two tiles each)
+
+// Operand layout of v_mfma_f32_32x32x16: lane l = 32*kg + i holds 8 consecutive k (8*kg .. +7 of
+// the 16-column step) of row/column i.  A 32-row weight block is two tiles (rows 0-15, 16-31);
+// in a tile, lane slot 16*c + r holds columns 8*c .. +7 of each 32-column sub-block, so lane
+// (kg, i) takes slot 16*kg + i%16 of tile i/16 for the first 16 columns of every sub-block
+// ("lo" registers) and slot 16*(kg+2) + i%16 for the second 16 columns ("hi" registers).
 template <int QT, typename AT>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                         AT *__restrict__ y, int M, int N, int K, int xcd_m) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
-    // x block in operand order: [sub-step s (4)][m-block (MB)][lane (64)] x 16 bytes, two buffers
-    __shared__ __attribute__((aligned(16))) uint8_t xs0[4 * MB * 1024];
-    __shared__ __attribute__((aligned(16))) uint8_t xs1[4 * MB * 1024];
+    // x block in operand order: [16-column step ks (8)][32-row block (MB32)][lane (64)] x 16 bytes
+    __shared__ __attribute__((aligned(16))) uint8_t xs0[8 * MB32 * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t xs1[8 * MB32 * 1024];
     __shared__ float lut[16];
     if constexpr (QT == QT_NF4) {
         if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODEBOOK[threadIdx.x];
     }
 
-
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = lane & 15, c = lane >> 4;
     const int G = K / TILE_COLS;
     const int n_tiles = N / TILE_ROWS;
 
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and each XCD has its own L2.  The
-    // output tiles are therefore dealt out so that one XCD owns a block of xm_band row-tiles by
-    // xn_band column-tiles: its L2 then only has to hold that band of x (re-read by every
+    // output tiles are therefore dealt out so that one XCD owns a block of band_m row-tiles by
+    // band_n column-tiles: its L2 then only has to hold that band of x (re-read by every
     // column-tile) and sees each weight tile from all its row-tiles at about the same time.
     const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int band_m = (tiles_m + xcd_m - 1) / xcd_m;            // row-tiles per XCD block
+    const int band_m = (tiles_m + xcd_m - 1) / xcd_m;
     const int xcd_n = 8 / xcd_m;
-    const int band_n = (tiles_n + xcd_n - 1) / xcd_n;            // column-tiles per XCD block
+    const int band_n = (tiles_n + xcd_n - 1) / xcd_n;
     const int tile_m = (xcd % xcd_m) * band_m + slot % band_m;
     const int tile_n = (xcd / xcd_m) * band_n + slot / band_m;
     if (slot >= band_m * band_n || tile_m >= tiles_m || tile_n >= tiles_n) return;   // whole workgroup leaves
     const int m0 = tile_m * GM;
     const int n0 = tile_n * GN + wave * GN_WAVE;
 
-    // weight tile rows of this wave (clamped: a tile row past N is computed and never stored)
-    const uint8_t *wt[NB];
+    // weight tiles of this lane: block nb covers rows n0 + 32*nb .. +31 (clamped: a tile row past N
+    // is computed and never stored)
+    const int kg = lane >> 5, i32 = lane & 31, r16 = lane & 15;
+    const int slot_lo = kg * 16 + r16, slot_hi = (kg + 2) * 16 + r16;
+    const uint8_t *wt[NB32];
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-        int trow = n0 / TILE_ROWS + nb;
+    for (int nb = 0; nb < NB32; nb++) {
+        int trow = n0 / TILE_ROWS + nb * 2 + (i32 >> 4);
         trow = trow < n_tiles ? trow : n_tiles - 1;
         wt[nb] = w + (int64_t)trow * G * F::TILE_BYTES;
     }
-    // x goes global -> registers -> LDS (operand order: chunk (s, mb) of lane l at
-    // ((s*MB + mb)*64 + l) * 16 bytes).  Wave w copies sub-step s = w of every m-block.
-    uint32_t xoff[MB];                                   // byte offset of this lane's chunk, per m-block
+
+    // x goes global -> registers -> LDS.  Per K step the workgroup copies 128 rows x 256 bytes;
+    // a wave-wide load covers 16 rows x 64 bytes: chunk = 4*wave + lane/16 (16 bytes each), row =
+    // 16*i + lane%16 for i = 0..7.  The chunk lands where the B operand wants it:
+    // step ks = chunk/2, kg = chunk%2, block row/32, lane slot 32*kg + row%32.
+    const int chunk = wave * 4 + (lane >> 4);
+    uint32_t xoff[8];
+    int xl[8];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        int row = m0 + mb * 16 + r;
+    for (int i = 0; i < 8; i++) {
+        const int row_in = i * 16 + r16;
+        int row = m0 + row_in;
         row = row < M ? row : M - 1;
-        xoff[mb] = (uint32_t)(((int64_t)row * K + wave * 32 + c * 8) * (int64_t)sizeof(AT));
+        xoff[i] = (uint32_t)(((int64_t)row * K + chunk * 8) * (int64_t)sizeof(AT));
+        xl[i] = (((chunk >> 1) * MB32 + (row_in >> 5)) * 64 + (chunk & 1) * 32 + (row_in & 31)) * 16;
     }
     const int last = G - 1;
-    auto load_x = [&](int kt, u32x4 (&xr)[MB]) {
+    auto load_x = [&](int kt, u32x4 (&xr)[8]) {
         kt = kt < last ? kt : last;                      // past the end: a harmless re-read, never used
         const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) xr[mb] = *(const u32x4 *)(xk + xoff[mb]);
+        for (int i = 0; i < 8; i++) xr[i] = *(const u32x4 *)(xk + xoff[i]);
     };
-    auto store_x = [&](uint8_t *buf, const u32x4 (&xr)[MB]) {
+    auto store_x = [&](uint8_t *buf, const u32x4 (&xr)[8]) {
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) *(u32x4 *)(buf + (wave * MB + mb) * 1024 + lane * 16) = xr[mb];
+        for (int i = 0; i < 8; i++) *(u32x4 *)(buf + xl[i]) = xr[i];
     };
-    auto load_w = [&](int kt, TileRegs<QT> (&t)[NB]) {
+    struct WRegs {
+        TileRegs<QT> lo[NB32], hi[NB32];
+    };
+    auto load_w = [&](int kt, WRegs &t) {
         kt = kt < last ? kt : last;
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) load_tile<QT>(wt[nb] + (int64_t)kt * F::TILE_BYTES, lane, r, t[nb]);
+        for (int nb = 0; nb < NB32; nb++) {
+            const uint8_t *tile = wt[nb] + (int64_t)kt * F::TILE_BYTES;
+            load_tile<QT>(tile, slot_lo, r16, t.lo[nb]);
+            t.hi[nb].q0 = *(const u32x4 *)(tile + slot_hi * 16);
+            if constexpr (F::BITS == 8) t.hi[nb].q1 = *(const u32x4 *)(tile + 1024 + slot_hi * 16);
+        }
     };
 
-    f32x4 acc[MB][NB];
+    f32x16 acc[MB32][NB32];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+    for (int mb = 0; mb < MB32; mb++)
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) acc[mb][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int nb = 0; nb < NB32; nb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[mb][nb][i] = 0.0f;
 
-    // 4 sub-steps of 32 columns, written in the order the hardware should issue them: after the
-    // MFMAs of an m-block, the x operand of that m-block for the NEXT sub-step is requested from
-    // LDS, and after every second MFMA one register pair of the next sub-step's weights is
-    // dequantized, so that LDS latency and the VALU work run in the shadow of the MFMA pipe.
-    auto compute = [&](const uint8_t *cur, const TileRegs<QT> (&tr)[NB]) {
-        V8 xv[MB];
-        u32x4 wv[NB];
+    // weights of 16-column step ks for block nb: sub-block ks/2, lo or hi registers
+    auto dequant_pair = [&](const WRegs &t, int ks, int nb, int p) -> uint32_t {
+        if (ks & 1) {
+            TileRegs<QT> h = t.hi[nb];
+            h.h = t.lo[nb].h;
+            return Dequant<QT, AT>::pair(h, ks >> 1, p, lut);
+        }
+        return Dequant<QT, AT>::pair(t.lo[nb], ks >> 1, p, lut);
+    };
+
+    // 8 steps of 16 columns, written in the order the hardware should issue them: after the MFMAs
+    // of an m-block its x operand for the NEXT step is requested from LDS, and a register pair of
+    // the next step's weights is dequantized after every MFMA, so that LDS latency and the VALU
+    // work run in the shadow of the MFMA pipe.
+    auto compute = [&](const uint8_t *cur, const WRegs &t) {
+        V8 xv[MB32];
+        u32x4 wv[NB32];
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) xv[mb] = *(const V8 *)(cur + mb * 1024 + lane * 16);
+        for (int mb = 0; mb < MB32; mb++) xv[mb] = *(const V8 *)(cur + mb * 1024 + lane * 16);
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
+        for (int nb = 0; nb < NB32; nb++)
 #pragma unroll
-            for (int p = 0; p < 4; p++) wv[nb][p] = Dequant<QT, AT>::pair(tr[nb], 0, p, lut);
+            for (int p = 0; p < 4; p++) wv[nb][p] = dequant_pair(t, 0, nb, p);
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-            u32x4 wn[NB];
+        for (int ks = 0; ks < 8; ks++) {
+            u32x4 wn[NB32];
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
+            for (int mb = 0; mb < MB32; mb++) {
 #pragma unroll
-                for (int nb = 0; nb < NB; nb++) {
+                for (int nb = 0; nb < NB32; nb++) {
                     mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
-                    if (s < 3 && (nb & 1)) {
-                        const int idx = mb * (NB / 2) + nb / 2;      // 0 .. 15: (weight block, pair)
-                        wn[idx >> 2][idx & 3] = Dequant<QT, AT>::pair(tr[idx >> 2], s + 1, idx & 3, lut);
+                    if (ks < 7) {
+                        const int idx = mb * NB32 + nb;           // 0 .. 7: (weight block, pair)
+                        wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);
                     }
                 }
-                if (s < 3) xv[mb] = *(const V8 *)(cur + ((s + 1) * MB + mb) * 1024 + lane * 16);
+                if (ks < 7) xv[mb] = *(const V8 *)(cur + ((ks + 1) * MB32 + mb) * 1024 + lane * 16);
+                // keep this order: the scheduler does not know how long an MFMA takes and would
+                // sink the LDS read down to its first use, exposing the LDS latency every time
+                __builtin_amdgcn_sched_barrier(0);
             }
-            if (s < 3) {
+            if (ks < 7) {
 #pragma unroll
-                for (int nb = 0; nb < NB; nb++) wv[nb] = wn[nb];
+                for (int nb = 0; nb < NB32; nb++) wv[nb] = wn[nb];
             }
         }
     };
@@ -267,8 +307,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
     // already in registers (it moves to LDS at the end of step kt) and the loads of step kt+2
     // are issued.  x rotates through two register sets, the weight tiles through three, hence
     // the period of six.
-    u32x4 xa[MB], xb[MB];
-    TileRegs<QT> w0[NB], w1[NB], w2[NB];
+    u32x4 xa[8], xb[8];
+    WRegs w0, w1, w2;
     load_x(0, xa);
     load_w(0, w0);
     load_x(1, xb);
@@ -295,22 +335,26 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
 #undef LOWBIT_GEMM_STEP
 
     // the MFMAs above are opaque to the compiler's hazard tracking: give the last results time
-    // to land before the accumulation registers are read back (an 8-pass MFMA needs 18 cycles)
-    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");
-    // C layout: lane = 16*g + col (col = x row within the m-block), register i = weight row 4*g + i
+    // to land before the accumulation registers are read back
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7");
+    // C layout of the 32x32 block: lane = 32*g + col (col = x row within the block), register i =
+    // weight row 8*(i/4) + 4*g + i%4: four consecutive n per group of registers
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        const int m = m0 + mb * 16 + r;
+    for (int mb = 0; mb < MB32; mb++) {
+        const int m = m0 + mb * 32 + i32;
         if (m < M) {
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                const int n = n0 + nb * 16 + c * 4;
-                if (n < N) {
-                    typedef AT at4 __attribute__((ext_vector_type(4)));
-                    at4 o;
+            for (int nb = 0; nb < NB32; nb++) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][i]);
-                    *(at4 *)(y + (int64_t)m * N + n) = o;
+                for (int q = 0; q < 4; q++) {
+                    const int n = n0 + nb * 32 + q * 8 + kg * 4;
+                    if (n < N) {
+                        typedef AT at4 __attribute__((ext_vector_type(4)));
+                        at4 o;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
+                        *(at4 *)(y + (int64_t)m * N + n) = o;
+                    }
                 }
             }
         }
