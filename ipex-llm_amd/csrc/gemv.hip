@@ -333,11 +333,22 @@ static int launch_gemv_t(const void *x, const void *w, void *y, int layout, int 
             const int mc = (M - m0) < 16 ? (M - m0) : 16;
             const AT *xp = (const AT *)x + (int64_t)m0 * K;
             AT *yp = (AT *)y + (int64_t)m0 * N;
-            if (mc == 1) launch_mfma<QT, AT, 1, 8, 2>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
-            else if (mc == 2) launch_mfma<QT, AT, 1, 8, 4>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
-            else if (mc <= 4) launch_mfma<QT, AT, 1, 8, 8>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
-            else if (mc <= 8) launch_mfma<QT, AT, 2, 4, 8>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
-            else launch_mfma<QT, AT, 4, 2, 8>(xp, (const uint8_t *)w, yp, mc, N, K, waves, st);
+            // Tiles per wave and round (U), measured on MI355X: 4 when K fits one round of 8 waves and
+            // there are many tile rows to spread over the CUs, else 2 with up to 16 waves and as many
+            // rounds as K needs.  XN = 16-byte chunks of x per lane = ceil(M * U / 4).
+            const bool u4 = (K / TILE_COLS) <= 32 && N >= 8192;
+            const uint8_t *wp = (const uint8_t *)w;
+            if (mc <= 4) {
+                if (u4) {
+                    if (mc == 1) launch_mfma<QT, AT, 1, 4, 1>(xp, wp, yp, mc, N, K, waves, st);
+                    else if (mc == 2) launch_mfma<QT, AT, 1, 4, 2>(xp, wp, yp, mc, N, K, waves, st);
+                    else launch_mfma<QT, AT, 1, 4, 4>(xp, wp, yp, mc, N, K, waves, st);
+                } else {
+                    if (mc <= 2) launch_mfma<QT, AT, 1, 2, 1>(xp, wp, yp, mc, N, K, waves, st);
+                    else launch_mfma<QT, AT, 1, 2, 2>(xp, wp, yp, mc, N, K, waves, st);
+                }
+            } else if (mc <= 8) launch_mfma<QT, AT, 2, 4, 8>(xp, wp, yp, mc, N, K, waves, st);
+            else launch_mfma<QT, AT, 4, 2, 8>(xp, wp, yp, mc, N, K, waves, st);
         }
         return 0;
     }
