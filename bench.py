@@ -216,6 +216,29 @@ def main():
             extra[f"sweep_M{m}"] = {"ms_per_step": round(ms2, 4),
                                     "GB/s": round(sweep_bytes(m) / (ms2 * 1e-3) / 1e9, 1)}
             del g2
+        # same sweep with q|k|v stored as one [12288 x 4096] weight and gate|up as one [22016 x 4096]
+        # (what the reference does by default: merged qkv_proj, fused gate/up): 4 launches per layer
+        merged = []
+        for mods in layers[:N_LAYERS]:
+            d = {name: blob for name, _, _, blob in mods}
+            # tile rows are contiguous in the tiled layout, so concatenating blobs concatenates rows
+            merged.append([("qkv", 12288, 4096, torch.cat([d["q"], d["k"], d["v"]])), ("o", 4096, 4096, d["o"]),
+                           ("gateup", 22016, 4096, torch.cat([d["gate"], d["up"]])),
+                           ("down", 4096, 11008, d["down"])])
+        ym = {"qkv": torch.empty((args.m, 12288), dtype=torch.float16, device=dev), "o": ys["o"],
+              "gateup": torch.empty((args.m, 22016), dtype=torch.float16, device=dev), "down": ys["down"]}
+
+        def sweep_merged():
+            st = stream()
+            for mods in merged:
+                for name, n, k, blob in mods:
+                    ggml.lowbit_forward(xs[k].data_ptr(), blob.data_ptr(), ym[name].data_ptr(), SYM_INT4,
+                                        ggml.LAYOUT_TILED, ggml.DT_F16, args.m, n, k, st)
+        g5 = capture(sweep_merged)
+        ms5 = time_graph(g5, max(5, args.steps // 2), 3)
+        extra["sweep_merged_qkv_gateup"] = {"ms_per_step": round(ms5, 4), "launches_per_step": 4 * N_LAYERS,
+                                            "GB/s": round(sweep_bytes(args.m) / (ms5 * 1e-3) / 1e9, 1)}
+        del merged, g5
         # prefill: one [11008 x 4096] linear at M = 2048
         m = 2048
         xp = torch.randn((m, 4096), generator=gen, device=dev, dtype=torch.float32).half()
