@@ -118,6 +118,17 @@ int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, in
 int lowbit_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
                 int64_t N, int64_t K, void *stream);
 
+/* Grouped product for mixture-of-experts layers, one launch for all experts.  The reference has
+ * no single call for it: it loops over the experts in Python and calls each expert's LowBitLinear
+ * on the rows routed to it (python/llm/src/ipex_llm/transformers/models/qwen2_moe.py:375-430 is the
+ * pattern).  Rows group_offsets[e] .. group_offsets[e+1]-1 of x [total_rows, K] are multiplied by
+ * the tiled weight w[e] [N, K]; y is [total_rows, N].  w (n_groups device pointers) and
+ * group_offsets (n_groups + 1 int32, ascending, group_offsets[n_groups] <= total_rows) live in
+ * DEVICE memory; total_rows is the host-side row count the grid is sized from. */
+int lowbit_grouped_forward(const void *x, const void *const *w, void *y, const int32_t *group_offsets,
+                           int n_groups, int64_t total_rows, int qtype, int act_dtype, int64_t N, int64_t K,
+                           void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,6 +15,8 @@ int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, in
                 int waves, hipStream_t st);
 int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 hipStream_t st);
+int launch_grouped_gemm(const void *x, const void *const *w, void *y, const int32_t *offsets, int n_groups,
+                        int total_rows, int qtype, int act_dtype, int N, int K, hipStream_t st);
 }  // namespace lowbit
 
 using namespace lowbit;
@@ -144,6 +146,20 @@ int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout,
     if (M <= 16 || layout != LOWBIT_LAYOUT_TILED)
         return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
     return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);
+}
+
+int lowbit_grouped_forward(const void *x, const void *const *w, void *y, const int32_t *group_offsets, int n_groups,
+                           int64_t total_rows, int qtype, int act_dtype, int64_t N, int64_t K, void *stream) {
+    if (int rc = check_weight_shape("lowbit_grouped_forward", qtype, N, K, LOWBIT_LAYOUT_TILED)) return rc;
+    if (n_groups < 0 || total_rows < 0 || total_rows > 0x7fffffff)
+        return fail(LOWBIT_EARG, "lowbit_grouped_forward: bad group count or row count");
+    if (act_dtype != LOWBIT_DT_F16 && act_dtype != LOWBIT_DT_BF16)
+        return fail(LOWBIT_EDTYPE, "lowbit_grouped_forward: activations must be f16 or bf16");
+    if (total_rows == 0 || n_groups == 0 || N == 0) return 0;
+    if (!x || !w || !y || !group_offsets || !aligned16(x) || (((uintptr_t)y) & 7))
+        return fail(LOWBIT_EARG, "lowbit_grouped_forward: null or misaligned pointer");
+    return check_launch(launch_grouped_gemm(x, w, y, group_offsets, n_groups, (int)total_rows, qtype, act_dtype, (int)N,
+                                            (int)K, (hipStream_t)stream), "lowbit_grouped_forward");
 }
 
 }  // extern "C"

@@ -165,7 +165,10 @@ constexpr int NB32 = GN_WAVE / 32;   // 32-row blocks of W per wave (two tiles e
 // ("lo" registers) and slot 16*(kg+2) + i%16 for the second 16 columns ("hi" registers).
 template <int QT, typename AT>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
-                                                        AT *__restrict__ y, int M, int N, int K, int xcd_m) {
+                                                        AT *__restrict__ y, int M, int N, int K, int xcd_m,
+                                                        const int32_t *__restrict__ group_offsets,
+                                                        const uint8_t *const *__restrict__ group_weights,
+                                                        int n_groups, int max_mtiles) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
     // x block in operand order: [16-column step ks (8)][32-row block (MB32)][lane (64)] x 16 bytes
@@ -184,15 +187,36 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
     // output tiles are therefore dealt out so that one XCD owns a block of band_m row-tiles by
     // band_n column-tiles: its L2 then only has to hold that band of x (re-read by every
     // column-tile) and sees each weight tile from all its row-tiles at about the same time.
-    const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int band_m = (tiles_m + xcd_m - 1) / xcd_m;
-    const int xcd_n = 8 / xcd_m;
-    const int band_n = (tiles_n + xcd_n - 1) / xcd_n;
-    const int tile_m = (xcd % xcd_m) * band_m + slot % band_m;
-    const int tile_n = (xcd / xcd_m) * band_n + slot / band_m;
-    if (slot >= band_m * band_n || tile_m >= tiles_m || tile_n >= tiles_n) return;   // whole workgroup leaves
-    const int m0 = tile_m * GM;
+    int m0, tile_n;
+    if (group_offsets == nullptr) {
+        const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        const int band_m = (tiles_m + xcd_m - 1) / xcd_m;
+        const int xcd_n = 8 / xcd_m;
+        const int band_n = (tiles_n + xcd_n - 1) / xcd_n;
+        const int tile_m = (xcd % xcd_m) * band_m + slot % band_m;
+        tile_n = (xcd / xcd_m) * band_n + slot / band_m;
+        if (slot >= band_m * band_n || tile_m >= tiles_m || tile_n >= tiles_n) return;   // whole workgroup leaves
+        m0 = tile_m * GM;
+    } else {
+        // Grouped mode (mixture-of-experts): rows group_offsets[e] .. group_offsets[e+1]-1 of x use
+        // weight group_weights[e].  The grid is sized on the host from an upper bound of row tiles;
+        // every workgroup finds its group by walking the offsets (a handful of scalar loads).
+        const int mt = blockIdx.x % max_mtiles;
+        tile_n = blockIdx.x / max_mtiles;
+        int e = 0, base = 0, r0 = 0, r1 = 0;
+        for (; e < n_groups; e++) {
+            r0 = group_offsets[e];
+            r1 = group_offsets[e + 1];
+            const int t = (r1 - r0 + GM - 1) / GM;
+            if (mt < base + t) break;
+            base += t;
+        }
+        if (e == n_groups) return;                                                  // whole workgroup leaves
+        m0 = r0 + (mt - base) * GM;
+        M = r1;                                     // rows past the group's end are clamped / not stored
+        w = group_weights[e];
+    }
     const int n0 = tile_n * GN + wave * GN_WAVE;
 
     // weight tiles of this lane: block nb covers rows n0 + 32*nb .. +31 (clamped: a tile row past N
@@ -370,8 +394,41 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     const int band_m = (tiles_m + xcd_m - 1) / xcd_m, band_n = (tiles_n + xcd_n - 1) / xcd_n;
     dim3 grid(8 * band_m * band_n);
     hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M,
-                       N, K, xcd_m);
+                       N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0);
     return 0;
+}
+
+template <int QT, typename AT>
+static int launch_grouped_t(const void *x, const void *const *w, void *y, const int32_t *offsets, int n_groups,
+                            int total_rows, int N, int K, hipStream_t st) {
+    const int max_mtiles = (total_rows + GM - 1) / GM + n_groups;    // every group adds at most one partial tile
+    const int tiles_n = (N + GN - 1) / GN;
+    hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT>), dim3(tiles_n * max_mtiles), dim3(256), 0, st, (const AT *)x,
+                       (const uint8_t *)nullptr, (AT *)y, 0, N, K, 1, offsets, (const uint8_t *const *)w, n_groups,
+                       max_mtiles);
+    return 0;
+}
+
+template <int QT>
+static int launch_grouped_q(const void *x, const void *const *w, void *y, const int32_t *offsets, int n_groups,
+                            int total_rows, int dt, int N, int K, hipStream_t st) {
+    if (dt == DT_F16) return launch_grouped_t<QT, _Float16>(x, w, y, offsets, n_groups, total_rows, N, K, st);
+    if (dt == DT_BF16) return launch_grouped_t<QT, __bf16>(x, w, y, offsets, n_groups, total_rows, N, K, st);
+    return -4;
+}
+
+// Grouped product for mixture-of-experts layers: one launch for all experts.
+int launch_grouped_gemm(const void *x, const void *const *w, void *y, const int32_t *offsets, int n_groups,
+                        int total_rows, int qtype, int act_dtype, int N, int K, hipStream_t st) {
+    if (total_rows == 0 || N == 0 || n_groups == 0) return 0;
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_grouped_q<QT_SYM_INT4>(x, w, y, offsets, n_groups, total_rows, act_dtype, N, K, st);
+    case QT_ASYM_INT4: return launch_grouped_q<QT_ASYM_INT4>(x, w, y, offsets, n_groups, total_rows, act_dtype, N, K, st);
+    case QT_SYM_INT8: return launch_grouped_q<QT_SYM_INT8>(x, w, y, offsets, n_groups, total_rows, act_dtype, N, K, st);
+    case QT_NF4: return launch_grouped_q<QT_NF4>(x, w, y, offsets, n_groups, total_rows, act_dtype, N, K, st);
+    case QT_FP8_E4M3: return launch_grouped_q<QT_FP8_E4M3>(x, w, y, offsets, n_groups, total_rows, act_dtype, N, K, st);
+    default: return -2;
+    }
 }
 
 template <int QT>

@@ -176,6 +176,16 @@ _lib.lowbit_gemm.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, 
 _lib.lowbit_gemm.restype = c_int
 
 
+_lib.lowbit_grouped_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int,
+                                        c_int64, c_int64, c_void_p]
+_lib.lowbit_grouped_forward.restype = c_int
+
+
+def lowbit_grouped_forward(x, w_ptrs, y, group_offsets, n_groups, total_rows, qtype, act_dtype, n, k, stream):
+    _check(_lib.lowbit_grouped_forward(x, w_ptrs, y, group_offsets, n_groups, total_rows, qtype, act_dtype,
+                                       n, k, stream), "lowbit_grouped_forward")
+
+
 def lowbit_blob_bytes(qtype, n_weights) -> int:
     return _lib.lowbit_blob_bytes(qtype, n_weights)
 

@@ -1,0 +1,92 @@
+"""Mixture-of-experts feed-forward on low-bit experts.
+
+The reference has no fused path for a Mixtral-style block at prefill: the Hugging Face block
+loops over the experts and calls each expert's (converted) LowBitLinear on the rows routed to
+it, then index_adds the weighted result (the same pattern as the reference's own
+transformers/models/qwen2_moe.py:375-430).  `moe_ffn_reference` is that loop;
+`moe_ffn_grouped` computes the same thing with three grouped launches (gate, up, down) over the
+rows sorted by expert.
+"""
+import ctypes
+
+import torch
+import torch.nn.functional as F
+
+import ipex_llm.ggml.model.llama.llama_cpp as ggml
+from ipex_llm.transformers.low_bit_linear import _DT, _as_u8, _stream
+from ipex_llm.utils.common import invalidInputError
+
+
+def route_top_k(router_logits: torch.Tensor, top_k: int = 2):
+    """softmax over experts in fp32, top-k, renormalised (Hugging Face Mixtral semantics)."""
+    probs = F.softmax(router_logits.float(), dim=-1)
+    weights, experts = torch.topk(probs, top_k, dim=-1)
+    weights = weights / weights.sum(dim=-1, keepdim=True)
+    return weights, experts
+
+
+class ExpertWeights:
+    """Device pointers of one projection of every expert ([N, K] tiled blobs of one qtype)."""
+
+    def __init__(self, linears):
+        invalidInputError(len(linears) > 0, "no experts")
+        l0 = linears[0]
+        self.qtype, self.out_len, self.in_len = l0.qtype, l0.out_len, l0.in_len
+        for lin in linears:
+            invalidInputError(lin.weight.device.type == "cuda" and lin.weight.quantized
+                              and (lin.qtype, lin.out_len, lin.in_len) == (self.qtype, self.out_len, self.in_len),
+                              "experts must be quantized, on the GPU and of one shape / qtype")
+        invalidInputError(ggml.lowbit_tileable(self.qtype, self.out_len, self.in_len),
+                          "grouped experts need out_features % 16 == 0 and in_features % 128 == 0")
+        self.blobs = [_as_u8(lin.weight.data) for lin in linears]        # keeps the storage alive
+        self.ptrs = torch.tensor([b.data_ptr() for b in self.blobs], dtype=torch.int64, device=l0.weight.device)
+
+
+def grouped_forward(x_sorted: torch.Tensor, group_offsets: torch.Tensor, experts: ExpertWeights):
+    """y[r] = x_sorted[r] @ dequant(W[e])^T for group_offsets[e] <= r < group_offsets[e+1]."""
+    invalidInputError(x_sorted.dim() == 2 and x_sorted.shape[1] == experts.in_len and x_sorted.dtype in _DT
+                      and x_sorted.dtype != torch.float32, "x must be [rows, K] in fp16 / bf16")
+    invalidInputError(group_offsets.dtype == torch.int32 and group_offsets.numel() == len(experts.blobs) + 1
+                      and group_offsets.device == x_sorted.device, "group_offsets must be int32 [E + 1] on the GPU")
+    x_sorted = x_sorted.contiguous()
+    rows = x_sorted.shape[0]
+    y = torch.empty((rows, experts.out_len), dtype=x_sorted.dtype, device=x_sorted.device)
+    if rows:
+        with torch.cuda.device(x_sorted.device):
+            ggml.lowbit_grouped_forward(x_sorted.data_ptr(), experts.ptrs.data_ptr(), y.data_ptr(),
+                                        group_offsets.data_ptr(), len(experts.blobs), rows, experts.qtype,
+                                        _DT[x_sorted.dtype], experts.out_len, experts.in_len, _stream())
+    return y
+
+
+def moe_ffn_reference(hidden, router_logits, w1, w3, w2, top_k=2):
+    """The per-expert loop: w1/w3/w2 are lists of LowBitLinear (gate, up, down)."""
+    weights, experts = route_top_k(router_logits, top_k)
+    out = torch.zeros_like(hidden)
+    for e in range(len(w1)):
+        tok, slot = torch.where(experts == e)
+        if tok.numel() == 0:
+            continue
+        xe = hidden[tok]
+        he = F.silu(w1[e](xe)) * w3[e](xe)
+        ye = w2[e](he) * weights[tok, slot].unsqueeze(-1).to(hidden.dtype)
+        out.index_add_(0, tok, ye.to(hidden.dtype))
+    return out
+
+
+def moe_ffn_grouped(hidden, router_logits, g1: ExpertWeights, g3: ExpertWeights, g2: ExpertWeights, top_k=2):
+    """Same result with three grouped launches over the (token, expert) pairs sorted by expert."""
+    n_exp = len(g1.blobs)
+    weights, experts = route_top_k(router_logits, top_k)
+    flat_e = experts.reshape(-1)
+    order = torch.argsort(flat_e, stable=True)
+    tok = torch.div(order, top_k, rounding_mode="floor")
+    counts = torch.bincount(flat_e, minlength=n_exp)
+    offsets = torch.zeros(n_exp + 1, dtype=torch.int32, device=hidden.device)
+    offsets[1:] = torch.cumsum(counts, 0).to(torch.int32)
+    xs = hidden[tok]
+    h = F.silu(grouped_forward(xs, offsets, g1)) * grouped_forward(xs, offsets, g3)
+    y = grouped_forward(h, offsets, g2) * weights.reshape(-1)[order].unsqueeze(-1).to(hidden.dtype)
+    out = torch.zeros_like(hidden)
+    out.index_add_(0, tok, y)
+    return out

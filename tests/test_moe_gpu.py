@@ -1,0 +1,64 @@
+"""Grouped expert GEMM (BASELINE configs[4], scaled down) against the per-expert LowBitLinear
+loop that is the reference's behaviour, and against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import lowbit_oracle as orc
+from ipex_llm.ggml.quantize import ggml_tensor_qtype as Q
+from ipex_llm.transformers.low_bit_linear import FP4Params, LowBitLinear
+from ipex_llm.transformers.moe import (ExpertWeights, grouped_forward, moe_ffn_grouped, moe_ffn_reference,
+                                       route_top_k)
+from gpu_util import weights
+
+pytestmark = pytest.mark.gpu
+
+
+def _experts(n_exp, n, k, qtype, seed):
+    out, raw = [], []
+    for e in range(n_exp):
+        w = weights(seed + e, (n, k))
+        lin = LowBitLinear(k, n, qtype, bias=False)
+        lin.weight = FP4Params(torch.from_numpy(w), qtype=qtype).to("cuda")
+        out.append(lin.eval())
+        raw.append(w)
+    return out, raw
+
+
+@pytest.mark.parametrize("qname,dtype", [("fp8_e4m3", torch.bfloat16), ("sym_int4", torch.float16),
+                                         ("nf4", torch.bfloat16), ("sym_int8", torch.float16)])
+def test_grouped_forward_matches_oracle_per_group(qname, dtype):
+    qtype = Q[qname]
+    n_exp, n, k = 5, 272, 256
+    lins, raw = _experts(n_exp, n, k, qtype, 8000)
+    counts = [130, 0, 1, 17, 129]                      # empty group, single row, partial and full tiles
+    rows = sum(counts)
+    torch.manual_seed(1)
+    x = torch.randn(rows, k).to(dtype).cuda()
+    offs = torch.tensor(np.concatenate([[0], np.cumsum(counts)]), dtype=torch.int32, device="cuda")
+    y = grouped_forward(x, offs, ExpertWeights(lins)).float().cpu().numpy()
+    r0 = 0
+    for e, c in enumerate(counts):
+        if c:
+            blob = orc.quantize(raw[e], qtype)
+            want = orc.mul_mat_exact(blob, x[r0:r0 + c].float().cpu().numpy(), (n, k), qtype)
+            tol = 2e-3 if dtype == torch.float16 else 8e-3
+            assert np.abs(y[r0:r0 + c] - want).max() <= tol * np.abs(want).max(), (e, c)
+        r0 += c
+
+
+@pytest.mark.parametrize("qname,dtype", [("fp8_e4m3", torch.bfloat16), ("sym_int4", torch.float16)])
+def test_moe_ffn_grouped_equals_per_expert_loop(qname, dtype):
+    qtype = Q[qname]
+    n_exp, hidden, ffn, tokens = 8, 256, 512, 77
+    w1, _ = _experts(n_exp, ffn, hidden, qtype, 8100)
+    w3, _ = _experts(n_exp, ffn, hidden, qtype, 8200)
+    w2, _ = _experts(n_exp, hidden, ffn, qtype, 8300)
+    torch.manual_seed(2)
+    x = torch.randn(tokens, hidden).to(dtype).cuda()
+    logits = torch.randn(tokens, n_exp).cuda()
+    wts, exp = route_top_k(logits, 2)
+    assert torch.allclose(wts.sum(-1), torch.ones(tokens, device="cuda"))
+    ref = moe_ffn_reference(x, logits, w1, w3, w2).float()
+    got = moe_ffn_grouped(x, logits, ExpertWeights(w1), ExpertWeights(w3), ExpertWeights(w2)).float()
+    assert (got - ref).abs().max() <= 1e-2 * ref.abs().max()
