@@ -255,12 +255,100 @@ def main():
         extra["prefill_M2048_N11008_K4096"] = {"ms": round(ms4, 4), "TFLOP/s": round(flop / (ms4 * 1e-3) / 1e12, 1),
                                                "pct_f16_mfma_peak": round(100 * flop / (ms4 * 1e-3) / 1e12 /
                                                                           MFMA_F16_PEAK_TFLOPS, 2)}
+        del xp, yp, g4
+        extra.update(other_configs(ggml, torch, gen, dev, layers[0], capture, time_graph, stream))
         out["extra"] = extra
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(layers[0], args.m, ggml, torch)
 
     print(json.dumps(out))
+
+
+QT = {"sym_int4": 2, "asym_int4": 3, "sym_int8": 8, "nf4": 10, "fp8_e4m3": 15}
+QT_BYTES = {2: (18, 32), 3: (20, 32), 8: (34, 32), 10: (34, 64), 15: (132, 128)}
+
+
+def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream):
+    """The parity-test configurations of BASELINE.json timed once each (not the headline):
+    configs[2] prefill, configs[3] Llama-3-70B shapes in nf4 / sym_int8, configs[4] Mixtral experts."""
+    res = {}
+
+    def new_weight(n, k, qtype, std):
+        w = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * std
+        tb, qk = QT_BYTES[qtype]
+        blob = torch.empty(n * k // qk * tb, dtype=torch.uint8, device=dev)
+        ggml.lowbit_quantize(w.data_ptr(), blob.data_ptr(), qtype, n, k, ggml.LAYOUT_TILED, stream())
+        torch.cuda.synchronize()
+        return blob
+
+    def time_set(mods, qtype, dt, tdt, m, reps):
+        xs = {k: torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32).to(tdt)
+              for k in {k for _, k, _ in mods}}
+        ys = {n: torch.empty((m, n), dtype=tdt, device=dev) for n, _, _ in mods}
+
+        def run():
+            st = stream()
+            for n, k, blob in mods:
+                ggml.lowbit_forward(xs[k].data_ptr(), blob.data_ptr(), ys[n].data_ptr(), qtype, ggml.LAYOUT_TILED,
+                                    dt, m, n, k, st)
+        g = capture(run)
+        ms = time_graph(g, reps, 2)
+        flop = sum(2.0 * m * n * k for n, k, _ in mods)
+        byts = sum(b.numel() + 2 * m * (n + k) for n, k, b in mods)
+        return {"ms": round(ms, 4), "TFLOP/s": round(flop / ms / 1e9, 1), "GB/s": round(byts / ms / 1e6, 1)}
+
+    # configs[2]: one layer's 7 linears at M = 512 / 2048, sym_int4 and asym_int4, fp16
+    sym = [(n, k, b) for _, n, k, b in layer0]
+    asym = [(n, k, new_weight(n, k, QT["asym_int4"], 0.02)) for n, k, _ in sym]
+    for name, mods in (("sym_int4", sym), ("asym_int4", asym)):
+        for m in (512, 2048):
+            res[f"prefill_layer_{name}_M{m}"] = time_set(mods, QT[name], ggml.DT_F16, torch.float16, m, 5)
+    del asym
+    # configs[3]: Llama-3-70B linear set (q, k, v, gate, up, down), bf16
+    shapes70 = [(8192, 8192), (1024, 8192), (1024, 8192), (28672, 8192), (28672, 8192), (8192, 28672)]
+    for name in ("nf4", "sym_int8"):
+        mods = [(n, k, new_weight(n, k, QT[name], 0.015)) for n, k in shapes70]
+        for m in (1, 16, 1024):
+            res[f"llama3_70b_{name}_M{m}"] = time_set(mods, QT[name], ggml.DT_BF16, torch.bfloat16, m,
+                                                      5 if m > 16 else 20)
+        del mods
+    # configs[4]: Mixtral 8x7B expert FFN, fp8_e4m3, 512 tokens, top-2, bf16: three grouped launches
+    import torch.nn.functional as F
+    n_exp, hid, ffn, tokens = 8, 4096, 14336, 512
+    qt = QT["fp8_e4m3"]
+    blobs = {p: [new_weight(n, k, qt, 0.02) for _ in range(n_exp)]
+             for p, (n, k) in (("w1", (ffn, hid)), ("w3", (ffn, hid)), ("w2", (hid, ffn)))}
+    ptrs = {p: torch.tensor([b.data_ptr() for b in bl], dtype=torch.int64, device=dev) for p, bl in blobs.items()}
+    logits = torch.randn((tokens, n_exp), generator=gen, device=dev)
+    hidden = torch.randn((tokens, hid), generator=gen, device=dev).bfloat16()
+    prob, experts = torch.topk(F.softmax(logits, dim=-1), 2, dim=-1)
+    flat = experts.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    offsets = torch.zeros(n_exp + 1, dtype=torch.int32, device=dev)
+    offsets[1:] = torch.cumsum(torch.bincount(flat, minlength=n_exp), 0).to(torch.int32)
+    rows = tokens * 2
+    xs = hidden[order // 2].contiguous()
+    h1 = torch.empty((rows, ffn), dtype=torch.bfloat16, device=dev)
+    h3 = torch.empty((rows, ffn), dtype=torch.bfloat16, device=dev)
+    yo = torch.empty((rows, hid), dtype=torch.bfloat16, device=dev)
+
+    def moe():
+        st = stream()
+        ggml.lowbit_grouped_forward(xs.data_ptr(), ptrs["w1"].data_ptr(), h1.data_ptr(), offsets.data_ptr(), n_exp,
+                                    rows, qt, ggml.DT_BF16, ffn, hid, st)
+        ggml.lowbit_grouped_forward(xs.data_ptr(), ptrs["w3"].data_ptr(), h3.data_ptr(), offsets.data_ptr(), n_exp,
+                                    rows, qt, ggml.DT_BF16, ffn, hid, st)
+        ggml.lowbit_grouped_forward(h1.data_ptr(), ptrs["w2"].data_ptr(), yo.data_ptr(), offsets.data_ptr(), n_exp,
+                                    rows, qt, ggml.DT_BF16, hid, ffn, st)
+    g = capture(moe)
+    ms = time_graph(g, 10, 2)
+    flop = 2.0 * rows * 3 * ffn * hid
+    wb = sum(b.numel() for bl in blobs.values() for b in bl)
+    res["mixtral_moe_fp8_512tok_top2"] = {"ms": round(ms, 4), "TFLOP/s": round(flop / ms / 1e9, 1),
+                                          "weight_GB/s": round(wb / ms / 1e6, 1),
+                                          "rows_per_expert": [int(v) for v in (offsets[1:] - offsets[:-1]).tolist()]}
+    return res
 
 
 def cpu_baseline(mods, m, ggml, torch):
