@@ -14,6 +14,7 @@
 //   as the B operand (columns = m), so a lane ends up with groups of 4 consecutive n for one m
 //   and stores 8 contiguous bytes of y at a time.
 // FLOP per launch: 2*M*N*K; MFMA-bound (fp16 / bf16 dense peak).
+#include <type_traits>
 #include "lowbit_mfma.h"
 
 namespace lowbit {
@@ -163,8 +164,8 @@ constexpr int NB32 = GN_WAVE / 32;   // 32-row blocks of W per wave (two tiles e
 // in a tile, lane slot 16*c + r holds columns 8*c .. +7 of each 32-column sub-block, so lane
 // (kg, i) takes slot 16*kg + i%16 of tile i/16 for the first 16 columns of every sub-block
 // ("lo" registers) and slot 16*(kg+2) + i%16 for the second 16 columns ("hi" registers).
-template <int QT, typename AT>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+template <int QT, typename AT, bool DMA>
+__global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                         AT *__restrict__ y, int M, int N, int K, int xcd_m,
                                                         const int32_t *__restrict__ group_offsets,
                                                         const uint8_t *const *__restrict__ group_weights,
@@ -223,12 +224,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
     // is computed and never stored)
     const int kg = lane >> 5, i32 = lane & 31, r16 = lane & 15;
     const int slot_lo = kg * 16 + r16, slot_hi = (kg + 2) * 16 + r16;
-    const uint8_t *wt[NB32];
+    gbytes wt[NB32];
 #pragma unroll
     for (int nb = 0; nb < NB32; nb++) {
         int trow = n0 / TILE_ROWS + nb * 2 + (i32 >> 4);
         trow = trow < n_tiles ? trow : n_tiles - 1;
-        wt[nb] = w + (int64_t)trow * G * F::TILE_BYTES;
+        wt[nb] = (gbytes)w + (int64_t)trow * G * F::TILE_BYTES;
     }
 
     // x goes global -> registers -> LDS.  Per K step the workgroup copies 128 rows x 256 bytes;
@@ -236,17 +237,45 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
     // 16*i + lane%16 for i = 0..7.  The chunk lands where the B operand wants it:
     // step ks = chunk/2, kg = chunk%2, block row/32, lane slot 32*kg + row%32.
     const int chunk = wave * 4 + (lane >> 4);
-    uint32_t xoff[8];
-    int xl[8];
+    uint32_t xoff[DMA ? MB32 : 8];
+    int xl[DMA ? 1 : 8];
+    if constexpr (!DMA) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int row_in = i * 16 + r16;
-        int row = m0 + row_in;
-        row = row < M ? row : M - 1;
-        xoff[i] = (uint32_t)(((int64_t)row * K + chunk * 8) * (int64_t)sizeof(AT));
-        xl[i] = (((chunk >> 1) * MB32 + (row_in >> 5)) * 64 + (chunk & 1) * 32 + (row_in & 31)) * 16;
+        for (int i = 0; i < 8; i++) {
+            const int row_in = i * 16 + r16;
+            int row = m0 + row_in;
+            row = row < M ? row : M - 1;
+            xoff[i] = (uint32_t)(((int64_t)row * K + chunk * 8) * (int64_t)sizeof(AT));
+            xl[i] = (((chunk >> 1) * MB32 + (row_in >> 5)) * 64 + (chunk & 1) * 32 + (row_in & 31)) * 16;
+        }
+    } else {
+        // DMA form: x goes global -> LDS without passing through registers.  One wave-wide
+        // instruction fills one 1 KiB operand block (16-column step ks, 32-row block mb): lane
+        // 32*kg + i fetches the 16 bytes at row 32*mb + i, columns 16*ks + 8*kg, and the hardware
+        // writes the lanes to LDS in lane order.  Wave w fills blocks 8w .. 8w+7 (ks = 2w, 2w+1).
+#pragma unroll
+        for (int mb = 0; mb < MB32; mb++) {
+            int row = m0 + mb * 32 + i32;
+            row = row < M ? row : M - 1;
+            xoff[mb] = (uint32_t)(((int64_t)row * K + kg * 8) * (int64_t)sizeof(AT));
+        }
     }
     const int last = G - 1;
+    auto dma_x = [&](int kt, uint8_t *buf) {
+        kt = kt < last ? kt : last;
+        const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT) + wave * 2 * 16 * sizeof(AT);
+        // Issued from inline assembly: the compiler's wait-count pass treats an LDS-DMA as aliasing
+        // every later LDS access and would wait for it immediately.  Completion is awaited by the
+        // explicit vmcnt(0) ahead of the workgroup barrier that publishes the buffer.
+        const uint32_t lbase = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + wave * 8 * 1024);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint8_t *src = xk + xoff[DMA ? (j & 3) : 0] + (j >> 2) * 16 * sizeof(AT);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         :: "v"(src), "s"(lbase + j * 1024) : "memory", "m0");
+        }
+    };
     auto load_x = [&](int kt, u32x4 (&xr)[8]) {
         kt = kt < last ? kt : last;                      // past the end: a harmless re-read, never used
         const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
@@ -264,10 +293,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
         kt = kt < last ? kt : last;
 #pragma unroll
         for (int nb = 0; nb < NB32; nb++) {
-            const uint8_t *tile = wt[nb] + (int64_t)kt * F::TILE_BYTES;
+            const gbytes tile = wt[nb] + (int64_t)kt * F::TILE_BYTES;
             load_tile<QT>(tile, slot_lo, r16, t.lo[nb]);
-            t.hi[nb].q0 = *(const u32x4 *)(tile + slot_hi * 16);
-            if constexpr (F::BITS == 8) t.hi[nb].q1 = *(const u32x4 *)(tile + 1024 + slot_hi * 16);
+            t.hi[nb].q0 = ld<u32x4>(tile + slot_hi * 16);
+            if constexpr (F::BITS == 8) t.hi[nb].q1 = ld<u32x4>(tile + 1024 + slot_hi * 16);
         }
     };
 
@@ -290,14 +319,17 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
     };
 
     // 8 steps of 16 columns, written in the order the hardware should issue them: after the MFMAs
-    // of an m-block its x operand for the NEXT step is requested from LDS, and a register pair of
-    // the next step's weights is dequantized after every MFMA, so that LDS latency and the VALU
-    // work run in the shadow of the MFMA pipe.
-    auto compute = [&](const uint8_t *cur, const WRegs &t) {
-        V8 xv[MB32];
+    // of an m-block its x operand for the NEXT step is requested from LDS, and register pairs of
+    // the next step's weights are dequantized after every MFMA, so that LDS latency and the VALU
+    // work run in the shadow of the MFMA pipe.  MBC = number of 32-row blocks of x that take part
+    // (a compile-time constant: a branch around each MFMA would cut the schedule into pieces).
+    auto compute = [&](const uint8_t *cur, const WRegs &t, auto mbc_) {
+        constexpr int MBC = decltype(mbc_)::value;
+        constexpr int PER = (4 * NB32) / (MBC * NB32);        // dequantized pairs per MFMA slot
+        V8 xv[MBC];
         u32x4 wv[NB32];
 #pragma unroll
-        for (int mb = 0; mb < MB32; mb++) xv[mb] = *(const V8 *)(cur + mb * 1024 + lane * 16);
+        for (int mb = 0; mb < MBC; mb++) xv[mb] = *(const V8 *)(cur + mb * 1024 + lane * 16);
 #pragma unroll
         for (int nb = 0; nb < NB32; nb++)
 #pragma unroll
@@ -306,13 +338,16 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
         for (int ks = 0; ks < 8; ks++) {
             u32x4 wn[NB32];
 #pragma unroll
-            for (int mb = 0; mb < MB32; mb++) {
+            for (int mb = 0; mb < MBC; mb++) {
 #pragma unroll
                 for (int nb = 0; nb < NB32; nb++) {
                     mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
                     if (ks < 7) {
-                        const int idx = mb * NB32 + nb;           // 0 .. 7: (weight block, pair)
-                        wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);
+#pragma unroll
+                        for (int q = 0; q < PER; q++) {
+                            const int idx = (mb * NB32 + nb) * PER + q;   // 0 .. 4*NB32-1: (weight block, pair)
+                            wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);
+                        }
                     }
                 }
                 if (ks < 7) xv[mb] = *(const V8 *)(cur + ((ks + 1) * MB32 + mb) * 1024 + lane * 16);
@@ -326,7 +361,78 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
             }
         }
     };
+    typedef std::integral_constant<int, MB32> full_t;
 
+    auto epilogue = [&](auto mbc_) {
+        constexpr int MBC = decltype(mbc_)::value;
+    // the MFMAs above are opaque to the compiler's hazard tracking: give the last results time
+    // to land before the accumulation registers are read back
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7");
+    // C layout of the 32x32 block: lane = 32*g + col (col = x row within the block), register i =
+    // weight row 8*(i/4) + 4*g + i%4: four consecutive n per group of registers
+#pragma unroll
+    for (int mb = 0; mb < MBC; mb++) {
+        const int m = m0 + mb * 32 + i32;
+        if (m < M) {
+#pragma unroll
+            for (int nb = 0; nb < NB32; nb++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int n = n0 + nb * 32 + q * 8 + kg * 4;
+                    if (n < N) {
+                        typedef AT at4 __attribute__((ext_vector_type(4)));
+                        at4 o;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
+                        *(at4 *)(y + (int64_t)m * N + n) = o;
+                    }
+                }
+                // one 32x32 block at a time: moving all 128 accumulators to vector registers at
+                // once would set the register footprint of the whole kernel
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    };
+
+    if constexpr (DMA) {
+        // One K step ahead: while step kt is computed the x block of step kt+1 streams into the
+        // other LDS buffer and its weight tiles into the second register set.  The waits this
+        // leaves exposed are covered by the second workgroup that the smaller register footprint
+        // lets a CU hold.
+        auto run = [&](auto mbc) {
+            WRegs w0, w1;
+            dma_x(0, xs0);
+            load_w(0, w0);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            for (int kt = 0; kt + 1 < G; kt += 2) {
+                dma_x(kt + 1, xs1);
+                load_w(kt + 1, w1);
+                compute(xs0, w0, mbc);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                dma_x(kt + 2, xs0);                          // past the end: a clamped, unused re-read
+                load_w(kt + 2, w0);
+                compute(xs1, w1, mbc);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+            }
+            if (G & 1) compute(xs0, w0, mbc);
+        };
+        // tail tiles and small expert groups: 32-row blocks without rows of x skip their MFMAs
+        const int mb_cnt = (M - m0 + 31) / 32;
+        if (mb_cnt <= 1) {
+            run(std::integral_constant<int, 1>());
+            epilogue(std::integral_constant<int, 1>());
+        } else if (mb_cnt <= 2) {
+            run(std::integral_constant<int, 2>());
+            epilogue(std::integral_constant<int, 2>());
+        } else {
+            run(full_t());
+            epilogue(full_t());
+        }
+    } else {
     // Software pipeline, two K steps deep: while step kt is computed, the data of step kt+1 is
     // already in registers (it moves to LDS at the end of step kt) and the loads of step kt+2
     // are issued.  x rotates through two register sets, the weight tiles through three, hence
@@ -344,7 +450,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
     if (kt + (i) < G) {                                 \
         load_x(kt + (i) + 2, xld);                      \
         load_w(kt + (i) + 2, wl);                       \
-        compute(cur, wc);                               \
+        compute(cur, wc, full_t());                     \
         store_x(nxt, xst);                              \
         __syncthreads();                                \
     }
@@ -357,33 +463,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const AT *__restrict__ x
         LOWBIT_GEMM_STEP(5, xs1, xs0, xa, xb, w2, w1)
     }
 #undef LOWBIT_GEMM_STEP
-
-    // the MFMAs above are opaque to the compiler's hazard tracking: give the last results time
-    // to land before the accumulation registers are read back
-    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7");
-    // C layout of the 32x32 block: lane = 32*g + col (col = x row within the block), register i =
-    // weight row 8*(i/4) + 4*g + i%4: four consecutive n per group of registers
-#pragma unroll
-    for (int mb = 0; mb < MB32; mb++) {
-        const int m = m0 + mb * 32 + i32;
-        if (m < M) {
-#pragma unroll
-            for (int nb = 0; nb < NB32; nb++) {
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const int n = n0 + nb * 32 + q * 8 + kg * 4;
-                    if (n < N) {
-                        typedef AT at4 __attribute__((ext_vector_type(4)));
-                        at4 o;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
-                        *(at4 *)(y + (int64_t)m * N + n) = o;
-                    }
-                }
-            }
-        }
+    epilogue(full_t());
     }
 }
+
 
 template <int QT, typename AT>
 static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, int K, hipStream_t st) {
@@ -393,8 +476,17 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     const int xcd_n = 8 / xcd_m;
     const int band_m = (tiles_m + xcd_m - 1) / xcd_m, band_n = (tiles_n + xcd_n - 1) / xcd_n;
     dim3 grid(8 * band_m * band_n);
-    hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M,
-                       N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0);
+    // Two forms of the kernel.  The DMA form (x straight into LDS, one K step of prefetch, 128
+    // vector registers) lets a CU hold two workgroups that cover each other's waits; it wins as
+    // soon as there are more tiles than CUs.  With at most one tile per CU the register-staged
+    // form with its deeper prefetch is faster.
+    const bool dma = tiles_m * tiles_n > 256;
+    if (dma)
+        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
+                           (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0);
+    else
+        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, false>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
+                           (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0);
     return 0;
 }
 
@@ -403,7 +495,7 @@ static int launch_grouped_t(const void *x, const void *const *w, void *y, const 
                             int total_rows, int N, int K, hipStream_t st) {
     const int max_mtiles = (total_rows + GM - 1) / GM + n_groups;    // every group adds at most one partial tile
     const int tiles_n = (N + GN - 1) / GN;
-    hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT>), dim3(tiles_n * max_mtiles), dim3(256), 0, st, (const AT *)x,
+    hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true>), dim3(tiles_n * max_mtiles), dim3(256), 0, st, (const AT *)x,
                        (const uint8_t *)nullptr, (AT *)y, 0, N, K, 1, offsets, (const uint8_t *const *)w, n_groups,
                        max_mtiles);
     return 0;

@@ -31,17 +31,24 @@ template <int QT> struct TileRegs {
     u32x4 h;
 };
 
-template <int QT> __device__ inline void load_tile(const uint8_t *tile, int lane, int r, TileRegs<QT> &t) {
+// Loads through a pointer that is known to be global memory.  A pointer fetched from a table in
+// memory is generic to the compiler and would be read with flat loads, which also count against
+// the LDS wait counter.
+typedef const __attribute__((address_space(1))) uint8_t *gbytes;
+template <typename T> __device__ inline T ld(const uint8_t *p) { return *(const T *)p; }
+template <typename T> __device__ inline T ld(gbytes p) { return *(const __attribute__((address_space(1))) T *)p; }
+
+template <int QT, typename P> __device__ inline void load_tile(P tile, int lane, int r, TileRegs<QT> &t) {
     using F = Fmt<QT>;
-    t.q0 = *(const u32x4 *)(tile + lane * 16);
-    if constexpr (F::BITS == 8) t.q1 = *(const u32x4 *)(tile + 1024 + lane * 16);
+    t.q0 = ld<u32x4>(tile + lane * 16);
+    if constexpr (F::BITS == 8) t.q1 = ld<u32x4>(tile + 1024 + lane * 16);
     if constexpr (QT == QT_SYM_INT4 || QT == QT_SYM_INT8) {
-        const u32x2 h = *(const u32x2 *)(tile + F::TILE_CODE_BYTES + r * 8);
+        const u32x2 h = ld<u32x2>(tile + F::TILE_CODE_BYTES + r * 8);
         t.h[0] = h[0]; t.h[1] = h[1];
     } else if constexpr (QT == QT_ASYM_INT4) {
-        t.h = *(const u32x4 *)(tile + F::TILE_CODE_BYTES + r * 16);
+        t.h = ld<u32x4>(tile + F::TILE_CODE_BYTES + r * 16);
     } else {
-        t.h[0] = *(const uint32_t *)(tile + F::TILE_CODE_BYTES + r * 4);
+        t.h[0] = ld<uint32_t>(tile + F::TILE_CODE_BYTES + r * 4);
     }
 }
 
