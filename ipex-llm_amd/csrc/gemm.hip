@@ -33,6 +33,21 @@ constexpr int GN = 256;          // weight rows per workgroup (4 waves)
 // slip a few VALU instructions between consecutive MFMAs.
 template <int QT, typename AT> struct Dequant;
 
+// What the dequantizers need besides the tile: the nf4 code book (LDS) and the exponent pattern
+// that is OR-ed onto 4-bit codes, held in a vector register.  As a literal it would share the
+// instruction's only constant slot with the nibble mask and v_and_or_b32 would fall apart into
+// an AND and an OR.
+struct DqCtx {
+    const void *lut;
+    uint32_t magic;
+};
+template <int QT, typename AT> __device__ inline uint32_t dq_magic() {
+    uint32_t r;
+    if constexpr (sizeof(AT) == 2 && __is_same(AT, _Float16)) asm("v_mov_b32 %0, 0x64006400" : "=v"(r));
+    else asm("v_mov_b32 %0, 0x43004300" : "=v"(r));
+    return r;
+}
+
 __device__ inline f16x2 h2(uint32_t bits16) {
     const uint32_t p = (bits16 & 0xffffu) | (bits16 << 16);
     return __builtin_bit_cast(f16x2, p);
@@ -44,7 +59,7 @@ template <> __device__ inline uint32_t pk2<_Float16>(float a, float b) { return 
 template <> __device__ inline uint32_t pk2<__bf16>(float a, float b) { return pk(bf16x2{(__bf16)a, (__bf16)b}); }
 
 template <> struct Dequant<QT_SYM_INT4, _Float16> {
-    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT4> &t, int s, int p, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT4> &t, int s, int p, const DqCtx &cx) {
         const uint32_t hb = t.h[s >> 1];
         const f16x2 d2 = h2((s & 1) ? (hb >> 16) : hb);
         const f16x2 k1032 = {(_Float16)1032.0f, (_Float16)1032.0f};
@@ -53,21 +68,21 @@ template <> struct Dequant<QT_SYM_INT4, _Float16> {
         const uint32_t v = (p & 2) ? (t.q0[s] >> 8) : t.q0[s];
         // exact q - 8 first (0x6400 | q is the half 1024 + q), one rounding in the multiply by d
         if (p & 1)
-            return pk(__builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k72) * d2);
-        return pk((__builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1032) * d2);
+            return pk(__builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, cx.magic)), k16th, -k72) * d2);
+        return pk((__builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, cx.magic)) - k1032) * d2);
     }
 };
 
 template <> struct Dequant<QT_ASYM_INT4, _Float16> {
-    __device__ static uint32_t pair(const TileRegs<QT_ASYM_INT4> &t, int s, int p, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_ASYM_INT4> &t, int s, int p, const DqCtx &cx) {
         const f16x2 d2 = h2(t.h[s]), m2 = h2(t.h[s] >> 16);
         const f16x2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
         const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
         const f16x2 k64 = {(_Float16)64.0f, (_Float16)64.0f};
         const uint32_t v = (p & 2) ? (t.q0[s] >> 8) : t.q0[s];
         f16x2 q;
-        if (p & 1) q = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k64);
-        else q = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1024;
+        if (p & 1) q = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, cx.magic)), k16th, -k64);
+        else q = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, cx.magic)) - k1024;
         return pk(__builtin_elementwise_fma(q, d2, m2));
     }
 };
@@ -75,12 +90,12 @@ template <> struct Dequant<QT_ASYM_INT4, _Float16> {
 // 4-bit integer codes with bf16 activations: bf16 has no packed arithmetic on gfx950, so the
 // weight is formed in fp32 ((128 + q) comes for free as a bit pattern) and rounded once.
 template <int QT> struct DequantInt4Bf16 {
-    __device__ static uint32_t pair(const TileRegs<QT> &t, int s, int p, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT> &t, int s, int p, const DqCtx &cx) {
         float d, mn;
         tile_scale<QT>(t, s, d, mn);
         const float off = (QT == QT_SYM_INT4) ? 136.0f : 128.0f;
         const float c = mn - off * d;
-        const uint32_t pr = and_or(t.q0[s] >> (4 * p), 0x000f000fu, 0x43004300u);   // bf16 pair 128+q
+        const uint32_t pr = and_or(t.q0[s] >> (4 * p), 0x000f000fu, cx.magic);   // bf16 pair 128+q
         const float lo = __builtin_bit_cast(float, pr << 16);
         const float hi = __builtin_bit_cast(float, pr & 0xffff0000u);
         return pk2<__bf16>(fmaf(lo, d, c), fmaf(hi, d, c));
@@ -96,7 +111,7 @@ __device__ inline uint32_t code_word8(const u32x4 &q0, const u32x4 &q1, int s, i
 }
 
 template <> struct Dequant<QT_SYM_INT8, _Float16> {
-    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT8> &t, int s, int p, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT8> &t, int s, int p, const DqCtx &cx) {
         const uint32_t hb = t.h[s >> 1];
         const f16x2 d2 = h2((s & 1) ? (hb >> 16) : hb);
         // byte ^ 0x80 = q + 128 (unsigned); 0x6400 | u is the half 1024 + u
@@ -108,7 +123,7 @@ template <> struct Dequant<QT_SYM_INT8, _Float16> {
 };
 
 template <> struct Dequant<QT_SYM_INT8, __bf16> {
-    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT8> &t, int s, int p, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_SYM_INT8> &t, int s, int p, const DqCtx &cx) {
         float d, mn;
         tile_scale<QT_SYM_INT8>(t, s, d, mn);
         // byte ^ 0x80 = q + 128 as an unsigned byte, converted exactly; (u - 128) * d is one fp32
@@ -121,7 +136,7 @@ template <> struct Dequant<QT_SYM_INT8, __bf16> {
 
 // fp8: exact hardware conversion to fp32, fp32 product with the block scale, one rounding
 template <typename AT> struct Dequant<QT_FP8_E4M3, AT> {
-    __device__ static uint32_t pair(const TileRegs<QT_FP8_E4M3> &t, int s, int p, const void *) {
+    __device__ static uint32_t pair(const TileRegs<QT_FP8_E4M3> &t, int s, int p, const DqCtx &cx) {
         typedef float f32x2 __attribute__((ext_vector_type(2)));
         const float sc = __builtin_bit_cast(float, t.h[0]);
         const uint32_t w = code_word8(t.q0, t.q1, s, p);
@@ -133,8 +148,8 @@ template <typename AT> struct Dequant<QT_FP8_E4M3, AT> {
 // nf4: fp32 code book in LDS, one rounding after the scale.  Nibble order 0,2,4,6,1,3,5,7:
 // columns 2p and 2p+1 sit in nibbles p and p+4.
 template <typename AT> struct Dequant<QT_NF4, AT> {
-    __device__ static uint32_t pair(const TileRegs<QT_NF4> &t, int s, int p, const void *lut_) {
-        const float *lut = (const float *)lut_;
+    __device__ static uint32_t pair(const TileRegs<QT_NF4> &t, int s, int p, const DqCtx &cx) {
+        const float *lut = (const float *)cx.lut;
         const float d = h2f((s >> 1) ? (t.h[0] >> 16) : (t.h[0] & 0xffff));
         const uint32_t v = t.q0[s] >> (4 * p);
         return pk2<AT>(lut[v & 0xf] * d, lut[(v >> 16) & 0xf] * d);
@@ -308,14 +323,15 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mb][nb][i] = 0.0f;
 
+    const DqCtx ctx = {lut, dq_magic<QT, AT>()};
     // weights of 16-column step ks for block nb: sub-block ks/2, lo or hi registers
     auto dequant_pair = [&](const WRegs &t, int ks, int nb, int p) -> uint32_t {
         if (ks & 1) {
             TileRegs<QT> h = t.hi[nb];
             h.h = t.lo[nb].h;
-            return Dequant<QT, AT>::pair(h, ks >> 1, p, lut);
+            return Dequant<QT, AT>::pair(h, ks >> 1, p, ctx);
         }
-        return Dequant<QT, AT>::pair(t.lo[nb], ks >> 1, p, lut);
+        return Dequant<QT, AT>::pair(t.lo[nb], ks >> 1, p, ctx);
     };
 
     // 8 steps of 16 columns, written in the order the hardware should issue them: after the MFMAs
