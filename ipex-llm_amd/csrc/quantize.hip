@@ -43,30 +43,30 @@ template <int W> __device__ inline float group_first_absmax_signed(const float4 
     return mx;
 }
 
-__device__ inline uint32_t nf4_index(float v) {
+// Index of the code-book entry nearest to v (ties to the smaller index) = number of midpoints
+// below v.  The 15 midpoints (fp32 sums halved, as the reference computes them) sit in LDS and are
+// searched by bisection: 4 compares per element instead of 15.
+__device__ inline void nf4_fill_mids(float *mids) {
+    if (threadIdx.x < 15)
+        mids[threadIdx.x] = __fmul_rn(__fadd_rn(NF4_CODEBOOK[threadIdx.x], NF4_CODEBOOK[threadIdx.x + 1]), 0.5f);
+    __syncthreads();
+}
+__device__ inline uint32_t nf4_index(float v, const float *mids) {
     uint32_t idx = 0;
 #pragma unroll
-    for (int i = 0; i < 15; i++) {
-        const float mid = __fmul_rn(__fadd_rn(NF4_CODEBOOK[i], NF4_CODEBOOK[i + 1]), 0.5f);
-        idx += (v > mid) ? 1u : 0u;
-    }
+    for (int step = 8; step > 0; step >>= 1) idx += (v > mids[idx + step - 1]) ? step : 0;
     return idx;
 }
 
-template <int QT, int LAYOUT>
-__global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__ src, uint8_t *__restrict__ dst,
-                                                       int64_t n_blocks, int64_t K) {
+// Header bits and the four codes (one per byte) of this lane's float4; the LPB lanes of a block
+// cooperate through shuffles.
+template <int QT>
+__device__ inline void block_codes(const float4 &v, int lib, uint32_t &hdr, uint32_t &mine, const float *mids) {
     using F = Fmt<QT>;
-    constexpr int LPB = F::QK / 4;                       // lanes per block
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t blk = t / LPB;
-    const int lib = (int)(t % LPB);
-    if (blk >= n_blocks) return;                         // whole LPB-groups leave together
-    const float4 v = *(const float4 *)(src + blk * F::QK + lib * 4);
+    constexpr int LPB = F::QK / 4;
     const float e[4] = {v.x, v.y, v.z, v.w};
-
-    uint32_t hdr = 0;
-    uint32_t mine = 0;                                   // byte i = code of element 4*lib + i
+    hdr = 0;
+    mine = 0;                                            // byte i = code of element 4*lib + i
     if constexpr (QT == QT_SYM_INT4) {
         const float mx = group_first_absmax_signed<LPB>(v, lib);
         const float d = __fdiv_rn(mx, -8.0f);
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__
         const float id = (amax != 0.0f) ? __fdiv_rn(1.0f, amax) : 0.0f;
         hdr = f2h(amax);
 #pragma unroll
-        for (int i = 0; i < 4; i++) mine |= nf4_index(__fmul_rn(e[i], id)) << (8 * i);
+        for (int i = 0; i < 4; i++) mine |= nf4_index(__fmul_rn(e[i], id), mids) << (8 * i);
     } else {
         const float amax = group_max<LPB>(fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3]))));
         const float s = __fdiv_rn(amax, 448.0f);
@@ -114,56 +114,113 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__
 #pragma unroll
         for (int i = 0; i < 4; i++) mine |= f32_to_e4m3(__fmul_rn(e[i], is)) << (8 * i);
     }
+}
 
-    const int64_t bpr = K / F::QK;                       // blocks per row
-    const int64_t n = blk / bpr;
-    const int kb = (int)(blk % bpr);
+// ggml layout: one thread group per block, written where the block lives.
+template <int QT>
+__global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__ src, uint8_t *__restrict__ dst,
+                                                       int64_t n_blocks) {
+    using F = Fmt<QT>;
+    constexpr int LPB = F::QK / 4;                       // lanes per block
+    __shared__ float mids[16];
+    if constexpr (QT == QT_NF4) nf4_fill_mids(mids);
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t blk = t / LPB;
+    const int lib = (int)(t % LPB);
+    if (blk >= n_blocks) return;                         // whole LPB-groups leave together
+    const float4 v = *(const float4 *)(src + blk * F::QK + lib * 4);
 
-    if constexpr (LAYOUT == LAYOUT_GGML) {
-        uint8_t *b = dst + blk * F::TS;
-        if (lib == 0) {
-            *(uint16_t *)b = (uint16_t)hdr;              // every block starts on an even address
-            if constexpr (F::HDR == 4) *(uint16_t *)(b + 2) = (uint16_t)(hdr >> 16);
-        }
-        if constexpr (F::BITS == 4) {
-            // byte j = code[j] | code[j + QK/2] << 4: lane i packs its own codes with lane i + LPB/2's
-            const uint32_t other = __shfl_down(mine, LPB / 2, LPB);
-            if (lib < LPB / 2) {
-                const uint32_t out = (mine & 0x0f0f0f0fu) | ((other & 0x0f0f0f0fu) << 4);
-                uint16_t *p = (uint16_t *)(b + F::HDR + lib * 4);
-                p[0] = (uint16_t)out;
-                p[1] = (uint16_t)(out >> 16);
-            }
-        } else {
+    uint32_t hdr, mine;
+    block_codes<QT>(v, lib, hdr, mine, mids);
+
+    uint8_t *b = dst + blk * F::TS;
+    if (lib == 0) {
+        *(uint16_t *)b = (uint16_t)hdr;              // every block starts on an even address
+        if constexpr (F::HDR == 4) *(uint16_t *)(b + 2) = (uint16_t)(hdr >> 16);
+    }
+    if constexpr (F::BITS == 4) {
+        // byte j = code[j] | code[j + QK/2] << 4: lane i packs its own codes with lane i + LPB/2's
+        const uint32_t other = __shfl_down(mine, LPB / 2, LPB);
+        if (lib < LPB / 2) {
+            const uint32_t out = (mine & 0x0f0f0f0fu) | ((other & 0x0f0f0f0fu) << 4);
             uint16_t *p = (uint16_t *)(b + F::HDR + lib * 4);
-            p[0] = (uint16_t)mine;
-            p[1] = (uint16_t)(mine >> 16);
+            p[0] = (uint16_t)out;
+            p[1] = (uint16_t)(out >> 16);
         }
     } else {
-        // lane pair (2c, 2c+1) of a 32-column sub-block holds columns 8c .. 8c+7
-        const int sb = kb * (F::QK / 32) + lib / 8;      // sub-block index in the row
-        const int c = (lib % 8) / 2;
-        const int r = (int)(n % TILE_ROWS), j = sb % 4;
-        uint8_t *tile = dst + tile_offset<QT>(n, K, sb);
-        if (lib == 0) {
-            uint8_t *h = tile + tile_hdr_offset<QT>(r, j);
-            if constexpr (F::HDR == 2) *(uint16_t *)h = (uint16_t)hdr;
-            else *(uint32_t *)h = hdr;
-        }
-        if constexpr (F::BITS == 4) {
-            const uint32_t other = __shfl_down(mine, 1, LPB);
-            if ((lib & 1) == 0) {
-                // mine = columns 0..3 (bytes 0..3), other = columns 4..7; nibble order 0,2,4,6,1,3,5,7
-                const uint32_t out = (mine & 0xf) | (((mine >> 16) & 0xf) << 4) | ((other & 0xf) << 8) |
-                                     (((other >> 16) & 0xf) << 12) | (((mine >> 8) & 0xf) << 16) |
-                                     (((mine >> 24) & 0xf) << 20) | (((other >> 8) & 0xf) << 24) |
-                                     (((other >> 24) & 0xf) << 28);
-                *(uint32_t *)(tile + (c * 16 + r) * 16 + j * 4) = out;
-            }
-        } else {
-            *(uint32_t *)(tile + (j / 2) * 1024 + (c * 16 + r) * 16 + (j % 2) * 8 + (lib & 1) * 4) = mine;
-        }
+        uint16_t *p = (uint16_t *)(b + F::HDR + lib * 4);
+        p[0] = (uint16_t)mine;
+        p[1] = (uint16_t)(mine >> 16);
     }
+}
+
+// Tiled layout, assembled in LDS.  A workgroup owns one tile row (16 rows of W) by QTW tiles
+// (QTW * 128 columns): wave w reads rows 4w .. 4w+3, 1 or 2 KiB of contiguous fp32 each, the
+// codes are placed into an LDS image of the tiles, and the image goes out with contiguous
+// 16-byte stores.  (Writing the 4-byte pieces straight to HBM costs about twice the bytes, since
+// the 16 rows of a tile would arrive from different workgroups at different times.)
+constexpr int QTW = 4;
+
+template <int QT>
+__global__ __launch_bounds__(256) void quantize_tiled_kernel(const float *__restrict__ src, uint8_t *__restrict__ dst,
+                                                             int64_t K) {
+    using F = Fmt<QT>;
+    constexpr int LPB = F::QK / 4;
+    __shared__ __attribute__((aligned(16))) uint8_t img[QTW * F::TILE_BYTES];
+    __shared__ float mids[16];
+    if constexpr (QT == QT_NF4) nf4_fill_mids(mids);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tiles_k = (int)(K / TILE_COLS);
+    const int t0 = blockIdx.x * QTW;                                 // first tile of this strip
+    const int nt = tiles_k - t0 < QTW ? tiles_k - t0 : QTW;          // tiles in this strip
+    const int64_t row0 = (int64_t)blockIdx.y * TILE_ROWS;
+    constexpr int PASSES = QTW * TILE_COLS / 256;                    // 256 columns per wave-wide load
+
+    float4 v[4][PASSES];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ps++) {
+            int col = ps * 256 + lane * 4;
+            col = col < nt * TILE_COLS ? col : 0;                    // past the strip: a valid re-read, not stored
+            v[i][ps] = *(const float4 *)(src + (row0 + wave * 4 + i) * K + (int64_t)t0 * TILE_COLS + col);
+        }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ps++) {
+            const int r = wave * 4 + i;
+            const int col = ps * 256 + lane * 4;
+            const int lib = lane % LPB;
+            uint32_t hdr, mine;
+            block_codes<QT>(v[i][ps], lib, hdr, mine, mids);
+            if (col >= nt * TILE_COLS) continue;                      // whole blocks leave together
+            uint8_t *tile = img + (col / TILE_COLS) * F::TILE_BYTES;
+            const int j = (col % TILE_COLS) / 32;                     // sub-block in the tile
+            const int c = (col % 32) / 8;                             // lane group of 8 columns
+            if (lib == 0) {
+                uint8_t *h = tile + tile_hdr_offset<QT>(r, j);
+                if constexpr (F::HDR == 2) *(uint16_t *)h = (uint16_t)hdr;
+                else *(uint32_t *)h = hdr;
+            }
+            if constexpr (F::BITS == 4) {
+                const uint32_t other = __shfl_down(mine, 1, LPB);
+                if ((lane & 1) == 0) {
+                    // mine = columns 0..3 (bytes 0..3), other = columns 4..7; nibble order 0,2,4,6,1,3,5,7
+                    const uint32_t out = (mine & 0xf) | (((mine >> 16) & 0xf) << 4) | ((other & 0xf) << 8) |
+                                         (((other >> 16) & 0xf) << 12) | (((mine >> 8) & 0xf) << 16) |
+                                         (((mine >> 24) & 0xf) << 20) | (((other >> 8) & 0xf) << 24) |
+                                         (((other >> 24) & 0xf) << 28);
+                    *(uint32_t *)(tile + (c * 16 + r) * 16 + j * 4) = out;
+                }
+            } else {
+                *(uint32_t *)(tile + (j / 2) * 1024 + (c * 16 + r) * 16 + (j % 2) * 8 + (lane & 1) * 4) = mine;
+            }
+        }
+    __syncthreads();
+    uint8_t *out = dst + ((int64_t)blockIdx.y * tiles_k + t0) * F::TILE_BYTES;
+    const int bytes = nt * F::TILE_BYTES;                             // a multiple of 16
+    for (int o = threadIdx.x * 16; o < bytes; o += 256 * 16) *(uint4 *)(out + o) = *(const uint4 *)(img + o);
 }
 
 template <int QT> static int launch_q(const float *src, void *dst, int64_t N, int64_t K, int layout, hipStream_t st) {
@@ -174,11 +231,13 @@ template <int QT> static int launch_q(const float *src, void *dst, int64_t N, in
     const int64_t grid = (threads + 255) / 256;
     if (grid > 0x7fffffff) return -3;
     if (layout == LAYOUT_GGML)
-        hipLaunchKernelGGL((quantize_kernel<QT, LAYOUT_GGML>), dim3((unsigned)grid), dim3(256), 0, st, src,
-                           (uint8_t *)dst, n_blocks, K);
-    else
-        hipLaunchKernelGGL((quantize_kernel<QT, LAYOUT_TILED>), dim3((unsigned)grid), dim3(256), 0, st, src,
-                           (uint8_t *)dst, n_blocks, K);
+        hipLaunchKernelGGL((quantize_kernel<QT>), dim3((unsigned)grid), dim3(256), 0, st, src, (uint8_t *)dst, n_blocks);
+    else {
+        const int64_t strips = (K / TILE_COLS + QTW - 1) / QTW, tile_rows = N / TILE_ROWS;
+        if (tile_rows > 65535) return -3;
+        hipLaunchKernelGGL((quantize_tiled_kernel<QT>), dim3((unsigned)strips, (unsigned)tile_rows), dim3(256), 0, st, src,
+                           (uint8_t *)dst, K);
+    }
     return 0;
 }
 
