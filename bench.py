@@ -239,6 +239,29 @@ def main():
         extra["sweep_merged_qkv_gateup"] = {"ms_per_step": round(ms5, 4), "launches_per_step": 4 * N_LAYERS,
                                             "GB/s": round(sweep_bytes(args.m) / (ms5 * 1e-3) / 1e9, 1)}
         del merged, g5
+        # same sweep with the gate and up projections fused into one launch that also applies
+        # SiLU(gate) * up (xe_linear.mlp_forward_xpu): 6 launches per layer
+        if args.m <= 4:
+            yg = torch.empty((args.m, 11008), dtype=torch.float16, device=dev)
+
+            def sweep_fused():
+                st = stream()
+                for mods in layers:
+                    d = {name: (n, k, blob) for name, n, k, blob in mods}
+                    for name in ("q", "k", "v", "o"):
+                        n, k, blob = d[name]
+                        ggml.lowbit_forward(xs[k].data_ptr(), blob.data_ptr(), ys[name].data_ptr(), SYM_INT4,
+                                            ggml.LAYOUT_TILED, ggml.DT_F16, args.m, n, k, st)
+                    ggml.lowbit_mlp_forward(xs[4096].data_ptr(), d["gate"][2].data_ptr(), d["up"][2].data_ptr(),
+                                            yg.data_ptr(), SYM_INT4, ggml.DT_F16, args.m, 11008, 4096, 0, st)
+                    n, k, blob = d["down"]
+                    ggml.lowbit_forward(xs[k].data_ptr(), blob.data_ptr(), ys["down"].data_ptr(), SYM_INT4,
+                                        ggml.LAYOUT_TILED, ggml.DT_F16, args.m, n, k, st)
+            g6 = capture(sweep_fused)
+            ms6 = time_graph(g6, max(5, args.steps // 2), 3)
+            extra["sweep_fused_gate_up"] = {"ms_per_step": round(ms6, 4), "launches_per_step": 6 * N_LAYERS,
+                                            "GB/s": round(sweep_bytes(args.m) / (ms6 * 1e-3) / 1e9, 1)}
+            del g6
         # prefill: one [11008 x 4096] linear at M = 2048
         m = 2048
         xp = torch.randn((m, 4096), generator=gen, device=dev, dtype=torch.float32).half()
@@ -250,7 +273,7 @@ def main():
                 ggml.lowbit_forward(xp.data_ptr(), b.data_ptr(), yp.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED,
                                     ggml.DT_F16, 2048, 11008, 4096, st)
         g4 = capture(prefill)
-        ms4 = time_graph(g4, 5, 2) / 8
+        ms4 = time_graph(g4, 10, 10) / 8                  # clocks settle after some tens of launches
         flop = 2.0 * m * 11008 * 4096
         extra["prefill_M2048_N11008_K4096"] = {"ms": round(ms4, 4), "TFLOP/s": round(flop / (ms4 * 1e-3) / 1e12, 1),
                                                "pct_f16_mfma_peak": round(100 * flop / (ms4 * 1e-3) / 1e12 /

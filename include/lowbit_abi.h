@@ -51,6 +51,11 @@ extern "C" {
 #define LOWBIT_DT_BF16 1
 #define LOWBIT_DT_F32 2
 
+/* activation of the gate branch in lowbit_mlp_forward (values of SILU / GELU in
+ * python/llm/src/ipex_llm/transformers/models/utils.py:30-31) */
+#define LOWBIT_ACT_SILU 0
+#define LOWBIT_ACT_GELU 1  /* tanh form, as in Gemma */
+
 /* error codes */
 #define LOWBIT_OK 0
 #define LOWBIT_EARG (-1)     /* null / misaligned pointer, negative size */
@@ -117,6 +122,17 @@ int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, in
                 int64_t N, int64_t K, int waves, void *stream);
 int lowbit_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
                 int64_t N, int64_t K, void *stream);
+
+/* xe_linear.dequantize_rows (python/llm/src/ipex_llm/transformers/embedding.py:218-221; signature
+ * xpu_ops.py:59-62): dst[i, :] = dequant(w)[rows[i], :] for i < n_rows, rows = int64 indices in
+ * device memory; an index outside [0, N) yields zeros.  dst is [n_rows, K] of out_dtype. */
+int lowbit_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, void *dst, int qtype, int64_t N,
+                           int64_t K, int layout, int out_dtype, void *stream);
+/* xe_linear.mlp_forward_xpu (python/llm/src/ipex_llm/transformers/models/common.py:145-158; signature
+ * xpu_ops.py:34-37): y[M, N] = act(x * Wg^T) .* (x * Wu^T) in one launch, both weights tiled [N, K],
+ * M <= 4 (the reference fuses at M == 1 only, models/utils.py:246-259). */
+int lowbit_mlp_forward(const void *x, const void *w_gate, const void *w_up, void *y, int qtype, int act_dtype,
+                       int64_t M, int64_t N, int64_t K, int act, void *stream);
 
 /* Grouped product for mixture-of-experts layers, one launch for all experts.  The reference has
  * no single call for it: it loops over the experts in Python and calls each expert's LowBitLinear

@@ -7,6 +7,10 @@
 #include <string.h>
 
 namespace lowbit {
+int launch_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, void *out, int qtype, int64_t N,
+                           int64_t K, int layout, int out_dtype, hipStream_t st);
+int launch_mlp_gemv(const void *x, const void *wg, const void *wu, void *y, int qtype, int act_dtype, int M, int N,
+                    int K, int act, hipStream_t st);
 int launch_quantize(const float *src, void *dst, int qtype, int64_t N, int64_t K, int layout, hipStream_t st);
 int launch_relayout(const void *src, void *dst, int qtype, int64_t N, int64_t K, int src_layout, hipStream_t st);
 int launch_dequantize(const void *w, void *out, int qtype, int64_t N, int64_t K, int layout, int out_dtype,
@@ -146,6 +150,30 @@ int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout,
     if (M <= 16 || layout != LOWBIT_LAYOUT_TILED)
         return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
     return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);
+}
+
+int lowbit_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, void *dst, int qtype, int64_t N,
+                           int64_t K, int layout, int out_dtype, void *stream) {
+    if (int rc = check_weight_shape("lowbit_dequantize_rows", qtype, N, K, layout)) return rc;
+    if (n_rows < 0) return fail(LOWBIT_EARG, "lowbit_dequantize_rows: negative row count");
+    if (n_rows * K == 0) return 0;
+    if (!w || !rows || !dst || !aligned16(w))
+        return fail(LOWBIT_EARG, "lowbit_dequantize_rows: null or misaligned pointer");
+    return check_launch(launch_dequantize_rows(w, rows, n_rows, dst, qtype, N, K, layout, out_dtype,
+                                               (hipStream_t)stream), "lowbit_dequantize_rows");
+}
+
+int lowbit_mlp_forward(const void *x, const void *w_gate, const void *w_up, void *y, int qtype, int act_dtype,
+                       int64_t M, int64_t N, int64_t K, int act, void *stream) {
+    if (int rc = check_mm("lowbit_mlp_forward", x, w_gate, y, qtype, LOWBIT_LAYOUT_TILED, act_dtype, M, N, K)) return rc;
+    if (act != LOWBIT_ACT_SILU && act != LOWBIT_ACT_GELU)
+        return fail(LOWBIT_EARG, "lowbit_mlp_forward: activation must be LOWBIT_ACT_SILU or LOWBIT_ACT_GELU");
+    if (M > 4) return fail(LOWBIT_ESIZE, "lowbit_mlp_forward: M must be at most 4 (decode)");
+    if (M * N == 0) return 0;
+    if (K == 0) return fail(LOWBIT_ESHAPE, "lowbit_mlp_forward: K == 0");
+    if (!w_up || !aligned16(w_up)) return fail(LOWBIT_EARG, "lowbit_mlp_forward: null or misaligned pointer");
+    return check_launch(launch_mlp_gemv(x, w_gate, w_up, y, qtype, act_dtype, (int)M, (int)N, (int)K, act,
+                                        (hipStream_t)stream), "lowbit_mlp_forward");
 }
 
 int lowbit_grouped_forward(const void *x, const void *const *w, void *y, const int32_t *group_offsets, int n_groups,

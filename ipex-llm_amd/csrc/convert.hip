@@ -79,54 +79,74 @@ template <> __device__ inline __bf16 from_f32<__bf16>(float v) { return (__bf16)
 
 template <int QT, int LAYOUT, typename OT>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict__ w, OT *__restrict__ out,
-                                                      int64_t N, int64_t K) {
+                                                      int64_t n_out, int64_t N, int64_t K,
+                                                      const int64_t *__restrict__ rows) {
+    // rows == nullptr: output row i is weight row i.  Otherwise output row i is weight row rows[i]
+    // (xe_linear.dequantize_rows, python/llm/src/ipex_llm/transformers/embedding.py:218-221); an
+    // index outside [0, N) gives a row of zeros.
     const int64_t sbpr = K / 32;
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= N * sbpr) return;
-    const int64_t n = t / sbpr;
+    if (t >= n_out * sbpr) return;
+    const int64_t i_out = t / sbpr;
+    const int64_t n = rows ? rows[i_out] : i_out;
     const int sb = (int)(t % sbpr);
+    if (n < 0 || n >= N) {
+        OT *o = out + i_out * K + (int64_t)sb * 32;
+#pragma unroll
+        for (int i = 0; i < 32; i++) o[i] = from_f32<OT>(0.0f);
+        return;
+    }
     SubBlock s;
     if constexpr (LAYOUT == LAYOUT_GGML) ggml_load_sub<QT>(w, n, K, sb, s);
     else tiled_load_sub<QT>(w, n, K, sb, s);
-    OT *o = out + n * K + (int64_t)sb * 32;
+    OT *o = out + i_out * K + (int64_t)sb * 32;
 #pragma unroll
     for (int i = 0; i < 32; i++) o[i] = from_f32<OT>(decode<QT>(s.code[i], s.d, s.m));
 }
 
 template <int QT, typename OT>
-static int launch_dq2(const void *w, void *out, int64_t N, int64_t K, int layout, hipStream_t st) {
-    const int64_t threads = N * (K / 32);
+static int launch_dq2(const void *w, void *out, int64_t N, int64_t K, int layout, hipStream_t st, const int64_t *rows,
+                      int64_t n_rows) {
+    const int64_t n_out = rows ? n_rows : N;
+    const int64_t threads = n_out * (K / 32);
     if (threads == 0) return 0;
     const int64_t grid = (threads + 255) / 256;
     if (grid > 0x7fffffff) return -3;
     if (layout == LAYOUT_GGML)
         hipLaunchKernelGGL((dequant_kernel<QT, LAYOUT_GGML, OT>), dim3((unsigned)grid), dim3(256), 0, st,
-                           (const uint8_t *)w, (OT *)out, N, K);
+                           (const uint8_t *)w, (OT *)out, n_out, N, K, rows);
     else
         hipLaunchKernelGGL((dequant_kernel<QT, LAYOUT_TILED, OT>), dim3((unsigned)grid), dim3(256), 0, st,
-                           (const uint8_t *)w, (OT *)out, N, K);
+                           (const uint8_t *)w, (OT *)out, n_out, N, K, rows);
     return 0;
 }
 
-template <int QT> static int launch_dq(const void *w, void *out, int64_t N, int64_t K, int layout, int dt, hipStream_t st) {
+template <int QT>
+static int launch_dq(const void *w, void *out, int64_t N, int64_t K, int layout, int dt, hipStream_t st,
+                     const int64_t *rows, int64_t n_rows) {
     switch (dt) {
-    case DT_F16: return launch_dq2<QT, _Float16>(w, out, N, K, layout, st);
-    case DT_BF16: return launch_dq2<QT, __bf16>(w, out, N, K, layout, st);
-    case DT_F32: return launch_dq2<QT, float>(w, out, N, K, layout, st);
+    case DT_F16: return launch_dq2<QT, _Float16>(w, out, N, K, layout, st, rows, n_rows);
+    case DT_BF16: return launch_dq2<QT, __bf16>(w, out, N, K, layout, st, rows, n_rows);
+    case DT_F32: return launch_dq2<QT, float>(w, out, N, K, layout, st, rows, n_rows);
     default: return -4;
+    }
+}
+
+int launch_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, void *out, int qtype, int64_t N,
+                           int64_t K, int layout, int out_dtype, hipStream_t st) {
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_dq<QT_SYM_INT4>(w, out, N, K, layout, out_dtype, st, rows, n_rows);
+    case QT_ASYM_INT4: return launch_dq<QT_ASYM_INT4>(w, out, N, K, layout, out_dtype, st, rows, n_rows);
+    case QT_SYM_INT8: return launch_dq<QT_SYM_INT8>(w, out, N, K, layout, out_dtype, st, rows, n_rows);
+    case QT_NF4: return launch_dq<QT_NF4>(w, out, N, K, layout, out_dtype, st, rows, n_rows);
+    case QT_FP8_E4M3: return launch_dq<QT_FP8_E4M3>(w, out, N, K, layout, out_dtype, st, rows, n_rows);
+    default: return -2;
     }
 }
 
 int launch_dequantize(const void *w, void *out, int qtype, int64_t N, int64_t K, int layout, int out_dtype,
                       hipStream_t st) {
-    switch (qtype) {
-    case QT_SYM_INT4: return launch_dq<QT_SYM_INT4>(w, out, N, K, layout, out_dtype, st);
-    case QT_ASYM_INT4: return launch_dq<QT_ASYM_INT4>(w, out, N, K, layout, out_dtype, st);
-    case QT_SYM_INT8: return launch_dq<QT_SYM_INT8>(w, out, N, K, layout, out_dtype, st);
-    case QT_NF4: return launch_dq<QT_NF4>(w, out, N, K, layout, out_dtype, st);
-    case QT_FP8_E4M3: return launch_dq<QT_FP8_E4M3>(w, out, N, K, layout, out_dtype, st);
-    default: return -2;
-    }
+    return launch_dequantize_rows(w, nullptr, 0, out, qtype, N, K, layout, out_dtype, st);
 }
 
 }  // namespace lowbit

@@ -142,15 +142,27 @@ template <typename AT> __device__ inline typename Vec8<AT>::type ones8() {
 // ------------------------------------------------------------ MFMA GEMV
 
 constexpr int GEMV_MAX_WAVES = 16;
+
+// activation of the gate branch: 0 = SiLU, 1 = GELU in its tanh form (what Gemma uses)
+__device__ inline float gate_act(float g, int act) {
+    if (act == 0) return g / (1.0f + __expf(-g));
+    const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
+    return 0.5f * g * (1.0f + t);
+}
 constexpr int GEMV_LDS_X_BUDGET = 64 * 1024;
 
 // One workgroup = one tile row (16 output columns).  Per round, wave w owns U consecutive
 // tiles along K: it first issues every weight load of the round (so the whole slice is in
 // flight at once), then copies its slice of x into a wave-private LDS region, then runs
 // 4*U MFMAs whose A operand comes from LDS.  Rounds repeat until K is covered.
-template <int QT, typename AT, int MT, int U, int XN>
+//
+// DUAL: the fused gate/up projection of a gated MLP (xe_linear.mlp_forward_xpu,
+// python/llm/src/ipex_llm/transformers/models/common.py:145-158): the workgroup walks the same
+// tile row of two weights with one copy of x and writes act(x Wg^T) * (x Wu^T).
+template <int QT, typename AT, int MT, int U, int XN, bool DUAL>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
-                                                         AT *__restrict__ y, int M, int N, int K) {
+                                                         const uint8_t *__restrict__ w2, AT *__restrict__ y, int M,
+                                                         int N, int K, int act) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
     constexpr bool IS4 = (F::BITS == 4);
@@ -160,7 +172,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     constexpr int SLICE = U * TILE_COLS;                    // columns of x per wave and round
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ float red[GEMV_MAX_WAVES][MT][64];
+    constexpr int NW = DUAL ? 2 : 1;                        // weights walked side by side
+    __shared__ float red[GEMV_MAX_WAVES][NW * MT][64];
     __shared__ AT lut[16];
     if constexpr (QT == QT_NF4) {
         if (threadIdx.x < 16) lut[threadIdx.x] = to_at<AT>(NF4_CODEBOOK[threadIdx.x]);
@@ -180,9 +193,10 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     AT *xs = (AT *)smem + (int64_t)wave * (XN * 512);       // [XN*64/(SLICE/8)][SLICE], private to this wave
     const AT *xa = xs + m_of_r * SLICE + 8 * c;
 
-    float acc[MT];
+    const uint8_t *wrow2 = DUAL ? w2 + (int64_t)blockIdx.x * G * F::TILE_BYTES : nullptr;
+    float acc[NW * MT];
 #pragma unroll
-    for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+    for (int i = 0; i < NW * MT; i++) acc[i] = 0.0f;
     const V8 ones = ones8<AT>();
     const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -205,11 +219,18 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
             xv[i] = *(const u32x4 *)(x + (int64_t)m * K + col);
         }
         __builtin_amdgcn_sched_barrier(0);                  // keep the x loads ahead of the weight loads
-        TileRegs<QT> tr[U];
+        TileRegs<QT> tr[NW * U];
 #pragma unroll
         for (int t = 0; t < U; t++) {
             const int g = gw + t;
             load_tile<QT>(wrow + (int64_t)(g < G ? g : G - 1) * F::TILE_BYTES, lane, r, tr[t]);
+        }
+        if constexpr (DUAL) {
+#pragma unroll
+            for (int t = 0; t < U; t++) {
+                const int g = gw + t;
+                load_tile<QT>(wrow2 + (int64_t)(g < G ? g : G - 1) * F::TILE_BYTES, lane, r, tr[U + t]);
+            }
         }
 
         __builtin_amdgcn_sched_barrier(0);
@@ -223,38 +244,42 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
         __builtin_amdgcn_wave_barrier();
 
 #pragma unroll
-        for (int t = 0; t < U; t++) {
-            const bool live = gw + t < G;
-            V8 a[4];
+        for (int wi = 0; wi < NW; wi++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) a[j] = *(const V8 *)(xa + (t * 4 + j) * 32);
+            for (int t = 0; t < U; t++) {
+                const TileRegs<QT> &tl = tr[wi * U + t];
+                const bool live = gw + t < G;
+                V8 a[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                V8 b;
-                if constexpr (IS4) b = Unpack<QT, AT>::run(tr[t].q0[j], lut);
-                else if (j < 2) b = Unpack8<QT, AT>::run(tr[t].q0[2 * j], tr[t].q0[2 * j + 1]);
-                else b = Unpack8<QT, AT>::run(tr[t].q1[2 * (j - 2)], tr[t].q1[2 * (j - 2) + 1]);
-                float d, mn;
-                tile_scale<QT>(tr[t], j, d, mn);
-                d = live ? d : 0.0f;
-                mn = live ? mn : 0.0f;
-                const f32x4 p = mfma16(a[j], b, zero4);
-                if constexpr (NEED_S) {
-                    const f32x4 s = mfma16(a[j], ones, zero4);
-                    const float e = mn - OFFSET * d;
+                for (int j = 0; j < 4; j++) a[j] = *(const V8 *)(xa + (t * 4 + j) * 32);
 #pragma unroll
-                    for (int i = 0; i < MT; i++) acc[i] = fmaf(e, s[i], fmaf(d, p[i], acc[i]));
-                } else {
+                for (int j = 0; j < 4; j++) {
+                    V8 b;
+                    if constexpr (IS4) b = Unpack<QT, AT>::run(tl.q0[j], lut);
+                    else if (j < 2) b = Unpack8<QT, AT>::run(tl.q0[2 * j], tl.q0[2 * j + 1]);
+                    else b = Unpack8<QT, AT>::run(tl.q1[2 * (j - 2)], tl.q1[2 * (j - 2) + 1]);
+                    float d, mn;
+                    tile_scale<QT>(tl, j, d, mn);
+                    d = live ? d : 0.0f;
+                    mn = live ? mn : 0.0f;
+                    const f32x4 p = mfma16(a[j], b, zero4);
+                    if constexpr (NEED_S) {
+                        const f32x4 s = mfma16(a[j], ones, zero4);
+                        const float e = mn - OFFSET * d;
 #pragma unroll
-                    for (int i = 0; i < MT; i++) acc[i] = fmaf(d, p[i], acc[i]);
+                        for (int i = 0; i < MT; i++)
+                            acc[wi * MT + i] = fmaf(e, s[i], fmaf(d, p[i], acc[wi * MT + i]));
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < MT; i++) acc[wi * MT + i] = fmaf(d, p[i], acc[wi * MT + i]);
+                    }
                 }
             }
-        }
     }
 
     // sum the K-slices of the waves; wave 0 writes.  C layout: lane = 16*grp + col, register i = row 4*grp + i.
 #pragma unroll
-    for (int i = 0; i < MT; i++) red[wave][i][lane] = acc[i];
+    for (int i = 0; i < NW * MT; i++) red[wave][i][lane] = acc[i];
     __syncthreads();
     if (wave == 0) {
         const int grp = lane >> 4, col = lane & 15;
@@ -262,6 +287,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
         for (int i = 0; i < MT; i++) {
             float s = 0.0f;
             for (int ww = 0; ww < W; ww++) s += red[ww][i][lane];
+            if constexpr (DUAL) {
+                float u = 0.0f;
+                for (int ww = 0; ww < W; ww++) u += red[ww][MT + i][lane];
+                s = gate_act(s, act) * u;
+            }
             const int m = grp * MT + i;
             if (m < M) y[(int64_t)m * N + (int64_t)blockIdx.x * 16 + col] = to_at<AT>(s);
         }
@@ -308,8 +338,9 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const AT *__restrict_
 
 // -------------------------------------------------------------- launch
 
-template <int QT, typename AT, int MT, int U, int XN>
-static void launch_mfma(const AT *x, const uint8_t *w, AT *y, int M, int N, int K, int waves, hipStream_t st) {
+template <int QT, typename AT, int MT, int U, int XN, bool DUAL = false>
+static void launch_mfma(const AT *x, const uint8_t *w, AT *y, int M, int N, int K, int waves, hipStream_t st,
+                        const uint8_t *w2 = nullptr, int act = 0) {
     const int G = K / TILE_COLS;
     // waves: enough that one round covers K, within the block size limit and the LDS budget for x
     int wv = (G + U - 1) / U;
@@ -319,8 +350,8 @@ static void launch_mfma(const AT *x, const uint8_t *w, AT *y, int M, int N, int 
     if (waves > 0 && waves < wv) wv = waves;
     if (wv < 1) wv = 1;
     const size_t lds = (size_t)wv * XN * 512 * sizeof(AT);
-    hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, MT, U, XN>), dim3(N / TILE_ROWS), dim3(64 * wv), lds, st, x, w, y, M, N,
-                       K);
+    hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, MT, U, XN, DUAL>), dim3(N / TILE_ROWS), dim3(64 * wv), lds, st, x, w, w2,
+                       y, M, N, K, act);
 }
 
 template <int QT, typename AT>
@@ -364,6 +395,39 @@ static int launch_gemv_q(const void *x, const void *w, void *y, int layout, int 
     if (dt == DT_F16) return launch_gemv_t<QT, _Float16>(x, w, y, layout, M, N, K, waves, st);
     if (dt == DT_BF16) return launch_gemv_t<QT, __bf16>(x, w, y, layout, M, N, K, waves, st);
     return -4;
+}
+
+template <int QT, typename AT>
+static int launch_mlp_t(const void *x, const void *wg, const void *wu, void *y, int M, int N, int K, int act,
+                        hipStream_t st) {
+    // two tiles of each weight per wave and round (as many registers as four tiles of one weight)
+    const AT *xp = (const AT *)x;
+    const uint8_t *g = (const uint8_t *)wg, *u = (const uint8_t *)wu;
+    if (M <= 2) launch_mfma<QT, AT, 1, 2, 1, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
+    else launch_mfma<QT, AT, 1, 2, 2, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
+    return 0;
+}
+
+template <int QT>
+static int launch_mlp_q(const void *x, const void *wg, const void *wu, void *y, int dt, int M, int N, int K, int act,
+                        hipStream_t st) {
+    if (dt == DT_F16) return launch_mlp_t<QT, _Float16>(x, wg, wu, y, M, N, K, act, st);
+    if (dt == DT_BF16) return launch_mlp_t<QT, __bf16>(x, wg, wu, y, M, N, K, act, st);
+    return -4;
+}
+
+// y[M, N] = act(x Wg^T) * (x Wu^T), M <= 4, both weights tiled [N, K]
+int launch_mlp_gemv(const void *x, const void *wg, const void *wu, void *y, int qtype, int act_dtype, int M, int N,
+                    int K, int act, hipStream_t st) {
+    if (M == 0 || N == 0) return 0;
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_mlp_q<QT_SYM_INT4>(x, wg, wu, y, act_dtype, M, N, K, act, st);
+    case QT_ASYM_INT4: return launch_mlp_q<QT_ASYM_INT4>(x, wg, wu, y, act_dtype, M, N, K, act, st);
+    case QT_SYM_INT8: return launch_mlp_q<QT_SYM_INT8>(x, wg, wu, y, act_dtype, M, N, K, act, st);
+    case QT_NF4: return launch_mlp_q<QT_NF4>(x, wg, wu, y, act_dtype, M, N, K, act, st);
+    case QT_FP8_E4M3: return launch_mlp_q<QT_FP8_E4M3>(x, wg, wu, y, act_dtype, M, N, K, act, st);
+    default: return -2;
+    }
 }
 
 int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,

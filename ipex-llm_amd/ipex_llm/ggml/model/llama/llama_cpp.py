@@ -186,6 +186,23 @@ def lowbit_grouped_forward(x, w_ptrs, y, group_offsets, n_groups, total_rows, qt
                                        n, k, stream), "lowbit_grouped_forward")
 
 
+_lib.lowbit_dequantize_rows.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int64, c_int, c_int,
+                                        c_void_p]
+_lib.lowbit_dequantize_rows.restype = c_int
+_lib.lowbit_mlp_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int64, c_int64,
+                                    c_int, c_void_p]
+_lib.lowbit_mlp_forward.restype = c_int
+
+
+def lowbit_dequantize_rows(w, rows, n_rows, dst, qtype, n, k, layout, out_dtype, stream):
+    _check(_lib.lowbit_dequantize_rows(w, rows, n_rows, dst, qtype, n, k, layout, out_dtype, stream),
+           "lowbit_dequantize_rows")
+
+
+def lowbit_mlp_forward(x, w_gate, w_up, y, qtype, act_dtype, m, n, k, act, stream):
+    _check(_lib.lowbit_mlp_forward(x, w_gate, w_up, y, qtype, act_dtype, m, n, k, act, stream), "lowbit_mlp_forward")
+
+
 def lowbit_blob_bytes(qtype, n_weights) -> int:
     return _lib.lowbit_blob_bytes(qtype, n_weights)
 

@@ -68,8 +68,11 @@ def _assign(model, name, tensor):
     if leaf in mod._parameters:
         old = mod._parameters[leaf]
         if isinstance(old, FP4Params):
+            shape = old._shape
+            if shape is None and hasattr(mod, "num_embeddings"):      # LowBitEmbedding skeleton
+                shape = torch.Size((mod.num_embeddings, mod.embedding_dim))
             mod._parameters[leaf] = FP4Params(tensor, requires_grad=False, quantized=True,
-                                              _shape=old._shape, qtype=old.qtype)
+                                              _shape=shape, qtype=old.qtype)
         else:
             mod._parameters[leaf] = torch.nn.Parameter(tensor, requires_grad=False)
     elif leaf in mod._buffers:
@@ -82,7 +85,7 @@ def unconverted_linears(state_dict):
     """Module names whose saved weight is still a dense matrix: they were excluded from the
     conversion when the model was saved and must be excluded again when it is rebuilt."""
     return [k[:-len(".weight")] for k, v in state_dict.items()
-            if k.endswith(".weight") and v.dim() == 2 and v.dtype != torch.uint8]
+            if k.endswith(".weight") and v.dim() == 2 and v.numel() > 0 and v.dtype != torch.uint8]
 
 
 def load_low_bit(model, model_path):

@@ -133,6 +133,11 @@ def _replace_with_low_bit_linear(model, qtype, modules_to_not_convert=None,
                 model._modules[name].requires_grad_(False)
                 module.weight = None
 
+        elif embedding_qtype is not None and type(module) == nn.Embedding:
+            # convert.py:726-729 of the reference
+            from ipex_llm.transformers.embedding import LowBitEmbedding
+            model._modules[name] = LowBitEmbedding.from_embedding(module, convert_shape_only, embedding_qtype)
+
         if len(list(module.children())) > 0:
             _, _flag = _replace_with_low_bit_linear(
                 module, qtype, modules_to_not_convert, convert_shape_only, cpu_embedding,
@@ -148,8 +153,40 @@ def _optimize_pre(model, qtype=None):
     return model    # q/k/v merging and friends: attention path, not built here
 
 
+def convert_forward(m, target_m, new_forward):
+    """Bind new_forward to every sub-module of class target_m (convert.py:1185-1193 of the reference)."""
+    from types import MethodType
+    if m.__class__ == target_m:
+        m.forward = MethodType(new_forward, m)
+    for _, sub_m in m.named_children():
+        convert_forward(sub_m, target_m, new_forward)
+
+
 def _optimize_post(model):
-    return model    # per-architecture forward patches: not built here
+    """Of the reference's per-architecture patches only the gated-MLP fusion belongs to the low-bit
+    linear path (its kernel is xe_linear.mlp_forward_xpu).  The reference wires it per model class
+    (convert.py:1298, 1720-1739 ...); here every `*MLP` module with low-bit gate / up / down
+    projections and a SiLU or tanh-GELU activation gets it."""
+    from ipex_llm.transformers.low_bit_linear import LowBitLinear
+    from ipex_llm.transformers.models.common import mlp_gelu_forward, mlp_silu_forward
+    seen = set()
+    for module in model.modules():
+        cls = module.__class__
+        if cls in seen or not cls.__name__.endswith("MLP"):
+            continue
+        projs = [getattr(module, n, None) for n in ("gate_proj", "up_proj", "down_proj")]
+        act = getattr(module, "act_fn", None)
+        if not all(isinstance(p, LowBitLinear) for p in projs) or act is None:
+            continue
+        act_name = act.__class__.__name__
+        if isinstance(act, nn.SiLU) or act_name in ("SiLUActivation", "SiLU"):
+            seen.add(cls)
+            convert_forward(model, cls, mlp_silu_forward)
+        elif (isinstance(act, nn.GELU) and act.approximate == "tanh") or act_name in ("PytorchGELUTanh", "GELUTanh",
+                                                                                      "NewGELUActivation"):
+            seen.add(cls)
+            convert_forward(model, cls, mlp_gelu_forward)
+    return model
 
 
 def ggml_convert_low_bit(model, qtype, optimize_model=True,
@@ -164,10 +201,8 @@ def ggml_convert_low_bit(model, qtype, optimize_model=True,
     if qtype in ggml_tensor_qtype.values():
         index = list(ggml_tensor_qtype.values()).index(qtype)
         logger.info(f"Converting the current model to {list(ggml_tensor_qtype.keys())[index]} format......")
-    invalidInputError(not cpu_embedding and embedding_qtype is None and imatrix_data is None
-                      and not mixed_precision,
-                      "cpu_embedding / embedding_qtype / imatrix / mixed_precision are outside "
-                      "the low-bit linear path built here")
+    invalidInputError(not cpu_embedding and imatrix_data is None and not mixed_precision,
+                      "cpu_embedding / imatrix / mixed_precision are outside the low-bit linear path built here")
     modules_to_not_convert = [] if modules_to_not_convert is None else modules_to_not_convert
 
     if optimize_model and not disable_optimize_pre:

@@ -264,6 +264,43 @@ def dequant(x: torch.Tensor, w: torch.Tensor, qtype: int, layout: int = None, sh
     return out
 
 
+def dequantize_rows(x: torch.Tensor, w: torch.Tensor, qtype: int, state_size: int, output_size: int,
+                    layout: int = None):
+    """xe_linear.dequantize_rows (embedding.py:218-221, xpu_ops.py:59-62): fp32 [*x.shape, state_size],
+    row i = dequantized row x[i] of the [output_size, state_size] weight."""
+    invalidInputError(x.device.type == _ACCEL and w.device == x.device,
+                      "dequantize_rows expects indices and weight on the same GPU")
+    invalidInputError(x.dtype in (torch.int64, torch.int32), "indices must be int64 or int32")
+    if layout is None:
+        layout = device_layout(qtype, (output_size, state_size))
+    w = _as_u8(w)
+    invalidInputError(w.numel() == ggml.lowbit_blob_bytes(qtype, output_size * state_size),
+                      "weight blob does not match [output_size, state_size]")
+    rows = x.contiguous().view(-1).to(torch.int64)
+    out = torch.empty((rows.numel(), state_size), dtype=torch.float32, device=x.device)
+    if rows.numel():
+        with torch.cuda.device(x.device):
+            ggml.lowbit_dequantize_rows(w.data_ptr(), rows.data_ptr(), rows.numel(), out.data_ptr(), qtype,
+                                        output_size, state_size, layout, ggml.DT_F32, _stream())
+    return out.view(*x.shape, state_size)
+
+
+def mlp_forward_xpu(x: torch.Tensor, weight1: torch.Tensor, weight2: torch.Tensor, batch_size: int,
+                    state_size: int, output_size: int, act_type: int, qtype: int):
+    """xe_linear.mlp_forward_xpu (models/common.py:152-156, xpu_ops.py:34-37):
+    act(x @ W1^T) * (x @ W2^T) in one launch; act_type 0 = SiLU, 1 = GELU (tanh form)."""
+    invalidInputError(x.dim() == 2 and x.shape == (batch_size, state_size) and x.device.type == _ACCEL,
+                      "mlp_forward_xpu expects x of shape [batch_size, state_size] on the GPU")
+    invalidInputError(ggml.lowbit_tileable(qtype, output_size, state_size),
+                      "mlp_forward_xpu needs output_size % 16 == 0 and state_size % 128 == 0")
+    xc = (x if x.dtype != torch.float32 else x.half()).contiguous()
+    y = torch.empty((batch_size, output_size), dtype=xc.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        ggml.lowbit_mlp_forward(xc.data_ptr(), _as_u8(weight1).data_ptr(), _as_u8(weight2).data_ptr(), y.data_ptr(),
+                                qtype, _DT[xc.dtype], batch_size, output_size, state_size, act_type, _stream())
+    return y if y.dtype == x.dtype else y.to(x.dtype)
+
+
 # ------------------------------------------------------------------ FP4Params
 
 class FP4Params(torch.nn.Parameter):

@@ -75,9 +75,9 @@ class _BaseAutoModelClass:
         torch_dtype = kwargs.pop("torch_dtype", None)
         embedding_qtype = kwargs.pop("embedding_qtype", None)
         invalidInputError(user_quantization_config is None and not speculative
-                          and pipeline_parallel_stages == 1 and embedding_qtype is None,
-                          "quantization_config / speculative / pipeline_parallel_stages / "
-                          "embedding_qtype are outside the low-bit linear path built here")
+                          and pipeline_parallel_stages == 1,
+                          "quantization_config / speculative / pipeline_parallel_stages "
+                          "are outside the low-bit linear path built here")
 
         if load_in_4bit or load_in_low_bit:
             if load_in_low_bit == "fp16":
@@ -94,6 +94,7 @@ class _BaseAutoModelClass:
             invalidInputError(q_k not in ["sym_int4_rtn", "sym_int8_rtn"],
                               f"The dtype {q_k} is specified for NPU and cannot be used on CPU and GPU")
             invalidInputError(kwargs.pop("imatrix", None) is None, "imatrix quantization is not supported")
+            kwargs["embedding_qtype"] = embedding_qtype
             model = cls.load_convert(q_k, optimize_model, *args, **kwargs)
         else:
             if torch_dtype is not None:
@@ -114,6 +115,12 @@ class _BaseAutoModelClass:
         disk_embedding = kwargs.pop("disk_embedding", False)
         mixed_precision = kwargs.pop("mixed_precision", False)
         disable_optimize_pre = kwargs.pop("disable_optimize_pre", False)
+        embedding_qtype = kwargs.pop("embedding_qtype", None)
+        if embedding_qtype is not None:
+            # the reference documents 'q2_k' / 'q4_k' here (model.py:148); any qtype with a kernel works
+            invalidInputError(embedding_qtype in ("sym_int4", "asym_int4", "sym_int8", "nf4", "fp8_e4m3"),
+                              f"embedding_qtype {embedding_qtype} has no MI355X kernel")
+            embedding_qtype = ggml_tensor_qtype[embedding_qtype]
         invalidInputError(not disk_embedding, "disk_embedding is outside the path built here")
         kwargs.pop('device_map', None)
         torch_dtype = kwargs.pop("torch_dtype", "auto")
@@ -131,6 +138,7 @@ class _BaseAutoModelClass:
                                      modules_to_not_convert=modules_to_not_convert,
                                      cpu_embedding=cpu_embedding,
                                      torch_dtype=torch_dtype,
+                                     embedding_qtype=embedding_qtype,
                                      mixed_precision=mixed_precision,
                                      disable_optimize_pre=disable_optimize_pre)
         model.config.update({"bigdl_transformers_low_bit": q_k, "bigdl_disk_embedding": False})
@@ -148,6 +156,9 @@ class _BaseAutoModelClass:
         optimize_model = kwargs.pop("optimize_model", True)
         modules_to_not_convert = kwargs.pop("modules_to_not_convert", None)
         torch_dtype = kwargs.pop("torch_dtype", "auto")
+        embedding_qtype = kwargs.pop("embedding_qtype", None)     # as in the reference (model.py:588)
+        if embedding_qtype is not None:
+            embedding_qtype = ggml_tensor_qtype[embedding_qtype]
         config = AutoConfig.from_pretrained(pretrained_model_name_or_path)
         low_bit = config.to_dict().get("bigdl_transformers_low_bit", None)
         invalidInputError(low_bit,
@@ -163,7 +174,8 @@ class _BaseAutoModelClass:
             model = cls.HF_Model.from_config(config)
         skip = list(modules_to_not_convert or []) + unconverted_linears(state_dict)
         model = ggml_convert_low_bit(model, qtype, optimize_model, device="meta",
-                                     convert_shape_only=True, modules_to_not_convert=skip)
+                                     convert_shape_only=True, modules_to_not_convert=skip,
+                                     embedding_qtype=embedding_qtype)
         keys_file = os.path.join(pretrained_model_name_or_path, "load_keys.json")
         if os.path.isfile(keys_file):
             with open(keys_file) as f:

@@ -1,0 +1,164 @@
+"""Fused gate/up projection (xe_linear.mlp_forward_xpu) and row-gather dequantization
+(xe_linear.dequantize_rows / LowBitEmbedding) against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+import lowbit_oracle as orc
+import ipex_llm.ggml.model.llama.llama_cpp as ggml
+from ipex_llm.ggml.quantize import ggml_tensor_qtype as Q
+from ipex_llm.transformers.embedding import LowBitEmbedding
+from ipex_llm.transformers.low_bit_linear import (FP4Params, LowBitLinear, dequantize_rows, mlp_forward_xpu)
+from ipex_llm.transformers.models.common import fuse_mlp_base, mlp_gelu_forward, mlp_silu_forward
+from ipex_llm.transformers.models.utils import GELU, SILU, mlp_fusion_check
+from gpu_util import ALL, NAMES, acts, dev_quantize, dev_relayout, weights
+
+pytestmark = pytest.mark.gpu
+
+
+def _silu(g):
+    return g / (1.0 + np.exp(-g))
+
+
+def _gelu_tanh(g):
+    return 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,act", [(1, SILU), (3, GELU), (4, SILU)])
+def test_mlp_forward_matches_the_exact_gated_product(qtype, dtype, m, act):
+    n, k = 304, 640                      # 19 tile rows, K not a multiple of a full round of waves
+    wg, wu = weights(9000 + qtype, (n, k)), weights(9100 + qtype, (n, k))
+    x = acts(9200 + m, m, k, dtype)
+    bg, bu = dev_quantize(wg, qtype, ggml.LAYOUT_TILED), dev_quantize(wu, qtype, ggml.LAYOUT_TILED)
+    y = mlp_forward_xpu(x.cuda(), bg, bu, m, k, n, act, qtype).float().cpu().numpy()
+    xf = x.float().numpy()
+    g = orc.mul_mat_exact(orc.quantize(wg, qtype), xf, (n, k), qtype)
+    u = orc.mul_mat_exact(orc.quantize(wu, qtype), xf, (n, k), qtype)
+    want = (_silu(g) if act == SILU else _gelu_tanh(g)) * u
+    tol = 2e-3 if dtype == torch.float16 else 8e-3       # one rounding of the result to fp16 / bf16
+    assert np.abs(y - want).max() <= tol * np.abs(want).max()
+
+
+def test_mlp_forward_rejects_what_it_cannot_fuse():
+    n, k = 32, 128
+    b = dev_quantize(weights(1, (n, k)), 2, ggml.LAYOUT_TILED)
+    x = acts(2, 5, k, torch.float16).cuda()
+    with pytest.raises(RuntimeError, match="at most 4"):
+        mlp_forward_xpu(x, b, b, 5, k, n, SILU, 2)
+    with pytest.raises(RuntimeError, match="activation"):
+        mlp_forward_xpu(x[:1], b, b, 1, k, n, 7, 2)
+
+
+class _GatedMlp(nn.Module):
+    def __init__(self, hidden, ffn, act):
+        super().__init__()
+        self.gate_proj = nn.Linear(hidden, ffn, bias=False)
+        self.up_proj = nn.Linear(hidden, ffn, bias=False)
+        self.down_proj = nn.Linear(ffn, hidden, bias=False)
+        self.act_fn = act
+
+    def forward(self, x):
+        return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+
+
+@pytest.mark.parametrize("low_bit,act,fwd", [("sym_int4", nn.SiLU(), mlp_silu_forward),
+                                             ("fp8_e4m3", nn.GELU(approximate="tanh"), mlp_gelu_forward)])
+def test_optimize_model_patches_gated_mlps_and_the_fused_path_agrees(low_bit, act, fwd):
+    from ipex_llm import optimize_model
+    torch.manual_seed(11)
+    ref = _GatedMlp(256, 512, act).eval()
+
+    class _Wrap(nn.Module):                      # the patch looks for classes named *MLP
+        def __init__(self, mlp):
+            super().__init__()
+            self.mlp = mlp
+
+        def forward(self, x):
+            return self.mlp(x)
+    _GatedMlp.__name__ = "ToyMLP"
+    try:
+        model = optimize_model(_Wrap(ref), low_bit=low_bit).to("cuda")
+        assert model.mlp.forward.__func__ is fwd
+        x1 = torch.randn(1, 1, 256).half().cuda()
+        x8 = torch.randn(2, 8, 256).half().cuda()
+        assert mlp_fusion_check(x1, Q[low_bit], False) and not mlp_fusion_check(x8, Q[low_bit], False)
+        with torch.no_grad():
+            fused = model(x1).float()
+            m = model.mlp
+            plain = m.down_proj(m.act_fn(m.gate_proj(x1)) * m.up_proj(x1)).float()
+            assert fused.shape == plain.shape == (1, 1, 256)
+            assert (fused - plain).abs().max() <= 1e-2 * plain.abs().max()
+            y8 = model(x8)                                       # too many rows: the unfused branch
+            assert y8.shape == (2, 8, 256)
+            assert torch.equal(y8, m.down_proj(m.act_fn(m.gate_proj(x8)) * m.up_proj(x8)))
+    finally:
+        _GatedMlp.__name__ = "_GatedMlp"
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("layout", [ggml.LAYOUT_GGML, ggml.LAYOUT_TILED])
+def test_dequantize_rows_is_bit_exact_and_zero_fills_bad_indices(qtype, layout):
+    n, k = 48, 256
+    w = weights(9300 + qtype, (n, k))
+    blob = dev_quantize(w, qtype, layout)
+    table = orc.dequantize(orc.quantize(w, qtype), qtype, (n, k))
+    idx = torch.tensor([[0, 47, 5], [5, 17, 31]], dtype=torch.int64)
+    got = dequantize_rows(idx.cuda(), blob, qtype, k, n, layout=layout)
+    assert got.dtype == torch.float32 and got.shape == (2, 3, k)
+    assert np.array_equal(got.cpu().numpy(), table[idx.numpy()])
+    bad = torch.tensor([3, -1, n, 7], dtype=torch.int32).cuda()
+    got = dequantize_rows(bad, blob, qtype, k, n, layout=layout).cpu().numpy()
+    assert np.array_equal(got[[0, 3]], table[[3, 7]]) and not got[[1, 2]].any()
+    assert dequantize_rows(torch.empty(0, dtype=torch.int64).cuda(), blob, qtype, k, n, layout=layout).shape == (0, k)
+
+
+@pytest.mark.parametrize("qname", ["sym_int4", "nf4", "fp8_e4m3"])
+def test_lowbit_embedding_looks_up_dequantized_rows(qname):
+    qtype = Q[qname]
+    torch.manual_seed(3)
+    emb = nn.Embedding(320, 128).half()
+    low = LowBitEmbedding.from_embedding(emb, False, qtype)
+    assert low.weight.numel() == 0 and not low.qweight.quantized
+    with pytest.raises(RuntimeError, match="only supports GPU"):
+        low(torch.tensor([1]))
+    low = low.to("cuda")
+    assert isinstance(low.qweight, FP4Params) and low.qweight.quantized and low.qweight.device.type == "cuda"
+    ids = torch.randint(0, 320, (2, 7))
+    out = low(ids.cuda())
+    assert out.dtype == torch.float16 and out.shape == (2, 7, 128)
+    w = emb.weight.detach().float().numpy()
+    table = orc.dequantize(orc.quantize(w, qtype), qtype, w.shape)
+    assert np.array_equal(out.float().cpu().numpy(), table[ids.numpy()].astype(np.float16).astype(np.float32))
+    # back on the CPU the blob is the ggml blob of the table
+    assert np.array_equal(low.to("cpu").qweight.data.view(torch.uint8).numpy(), orc.quantize(w, qtype))
+
+
+def test_from_pretrained_with_embedding_qtype_and_fused_mlp(tmp_path):
+    transformers = pytest.importorskip("transformers")
+    from ipex_llm.transformers import AutoModelForCausalLM
+    cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=4, vocab_size=320,
+                                   max_position_embeddings=64)
+    torch.manual_seed(5)
+    hf = transformers.LlamaForCausalLM(cfg).eval()
+    src = tmp_path / "fp"
+    hf.save_pretrained(str(src))
+    model = AutoModelForCausalLM.from_pretrained(str(src), load_in_low_bit="sym_int4", embedding_qtype="sym_int8",
+                                                 modules_to_not_convert=["lm_head"])
+    assert isinstance(model.model.embed_tokens, LowBitEmbedding)
+    assert model.model.layers[0].mlp.forward.__func__ is mlp_silu_forward
+    ids = torch.randint(0, 320, (1, 1))                       # one token: the fused MLP launch
+    with torch.no_grad():
+        want = hf(ids).logits
+        got = model.to("cuda")(ids.cuda()).logits.float().cpu()
+    assert (got - want).abs().mean() / want.abs().mean() < 0.2
+    out = tmp_path / "lowbit"
+    model.save_low_bit(str(out))
+    again = AutoModelForCausalLM.load_low_bit(str(out), embedding_qtype="sym_int8")
+    assert isinstance(again.model.embed_tokens, LowBitEmbedding)
+    with torch.no_grad():
+        got2 = again.to("cuda")(ids.cuda()).logits.float().cpu()
+    assert torch.equal(got, got2)
