@@ -400,11 +400,13 @@ static int launch_gemv_q(const void *x, const void *w, void *y, int layout, int 
 template <int QT, typename AT>
 static int launch_mlp_t(const void *x, const void *wg, const void *wu, void *y, int M, int N, int K, int act,
                         hipStream_t st) {
-    // two tiles of each weight per wave and round (as many registers as four tiles of one weight)
+    // four tiles of each weight per wave and round, 8 waves for K = 4096: measured equal to two
+    // tiles with twice the rounds and ahead of 16-wave workgroups, which pack badly onto a CU
     const AT *xp = (const AT *)x;
     const uint8_t *g = (const uint8_t *)wg, *u = (const uint8_t *)wu;
-    if (M <= 2) launch_mfma<QT, AT, 1, 2, 1, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
-    else launch_mfma<QT, AT, 1, 2, 2, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
+    if (M == 1) launch_mfma<QT, AT, 1, 4, 1, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
+    else if (M == 2) launch_mfma<QT, AT, 1, 4, 2, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
+    else launch_mfma<QT, AT, 1, 4, 4, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
     return 0;
 }
 
