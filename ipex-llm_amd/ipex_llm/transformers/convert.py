@@ -32,12 +32,78 @@ def is_lm_head(name, model_config, out_features):
     return name == "lm_head" or getattr(model_config, "vocab_size", None) == out_features
 
 
+def is_gptq_linear(module) -> bool:
+    """A 4-bit GPTQ / AWQ linear as AutoGPTQ's QuantLinear or AutoAWQ's WQLinear_GEMM lay it out.
+    The reference tests the classes of those packages (convert.py:98-105, 512-513); they are not a
+    dependency here, so the layer is recognised by its tensors."""
+    return (all(hasattr(module, a) for a in ("qweight", "qzeros", "scales", "group_size", "wf"))
+            and getattr(module, "bits", getattr(module, "w_bit", None)) == 4)
+
+
 def is_linear_module(module):
-    """(is_linear, (in_features, out_features, mp_group)) - plain nn.Linear only; the vLLM /
-    DeepSpeed / GPTQ / AWQ layer classes of the reference are not handled."""
+    """(is_linear, (in_features, out_features, mp_group)): nn.Linear and 4-bit GPTQ / AWQ layers; the
+    vLLM / DeepSpeed layer classes of the reference (convert.py:138-232) are not handled."""
     if isinstance(module, nn.Linear):
         return True, (module.in_features, module.out_features, None)
+    if is_gptq_linear(module):
+        inf = getattr(module, "infeatures", None) or module.in_features
+        outf = getattr(module, "outfeatures", None) or module.out_features
+        return True, (inf, outf, None)
     return False, (None, None, None)
+
+
+def _unpack_int32(packed: torch.Tensor, wf: torch.Tensor, axis: int) -> torch.Tensor:
+    """Splits every int32 of `packed` into len(wf) 4-bit values (shifts wf) along `axis`:
+    the size of that axis grows by len(wf), value j of word r lands at index r * len(wf) + j."""
+    n = wf.numel()
+    shape = [1] * (packed.dim() + 1)
+    shape[axis + 1] = n
+    vals = torch.bitwise_and(torch.bitwise_right_shift(packed.unsqueeze(axis + 1), wf.reshape(shape)), 15)
+    out_shape = list(packed.shape)
+    out_shape[axis] *= n
+    return vals.reshape(out_shape).to(torch.uint8)
+
+
+def convert_gptq(module, awq=False, llm_awq=False, act_order=False):
+    """Repacks a 4-bit GPTQ / AWQ layer into an asym_int4 (ggml Q4_1) blob without touching the codes
+    (reference: convert.py:379-453).  w[o, i] = scale[g, o] * (q[i, o] - zero[g, o]) becomes
+    q * d + m with d = scale and m = -(zero * scale), both fp16; GPTQ stores zero - 1.
+    Returns (blob uint8 1-D in the ggml layout, g_id_map or None)."""
+    bits = getattr(module, "bits", getattr(module, "w_bit", None))
+    invalidInputError(bits == 4, "only 4-bit GPTQ / AWQ layers map onto asym_int4")
+    group = int(module.group_size)
+    invalidInputError(group % 32 == 0, "group_size must be a multiple of the 32-weight block")
+    wf = module.wf.to(torch.int32).reshape(-1)
+    scales = module.scales
+    zeros = _unpack_int32(module.qzeros, wf, 1).to(torch.int16)             # [groups, out]
+    if not awq:
+        zeros = zeros + 1
+    if awq:
+        q = _unpack_int32(module.qweight, wf, 1)                              # [in, out] (llm-awq: [out, in])
+        if llm_awq:
+            q = q.t()
+    else:
+        q = _unpack_int32(module.qweight, wf, 0)                              # [in, out]
+    g_id_map = None
+    if act_order and not awq:
+        invalidInputError(module.g_idx.shape[0] == q.shape[0], "g_idx and weight shape mismatch")
+        _, g_id_map = torch.sort(module.g_idx)
+        q = q[g_id_map, :]
+    if llm_awq:
+        real = module.in_features // group
+        zeros, scales = zeros[:, :real].t(), scales[:, :real].t()
+    in_f, out_f = q.shape
+    zeros = zeros.reshape(-1, out_f)[: in_f // group]
+    scales = scales.reshape(-1, out_f)[: in_f // group]
+    # codes: [out, blocks, 32] -> byte j = code j | code j+16 << 4
+    qb = q.t().contiguous().reshape(out_f, in_f // 32, 2, 16)
+    codes = torch.bitwise_or(qb[:, :, 0, :], torch.bitwise_left_shift(qb[:, :, 1, :], 4))
+    # one (d, m) per 32-weight block: every group covers group / 32 consecutive blocks
+    d = scales.t().to(torch.float16).repeat_interleave(group // 32, dim=1).contiguous()   # [out, blocks]
+    z = zeros.t().to(torch.float16).repeat_interleave(group // 32, dim=1).contiguous()
+    m = -(z * d)
+    blob = torch.cat([d.unsqueeze(-1).view(torch.uint8), m.unsqueeze(-1).view(torch.uint8), codes], dim=-1)
+    return blob.reshape(-1), g_id_map
 
 
 def use_scale_search(model_config, qtype):
@@ -89,7 +155,29 @@ def _replace_with_low_bit_linear(model, qtype, modules_to_not_convert=None,
             optimize_lm_head = (is_lm_head(name, model_config, out_features)
                                 and os.environ.get("IPEX_LLM_LAST_LM_HEAD", None) != "0")
             new_linear = None
-            if qtype not in (ggml_tensor_qtype["fp16"], ggml_tensor_qtype["bf16"]):
+            if is_gptq_linear(module):
+                # convert.py:511-545 of the reference: the codes are kept, only the packing changes
+                invalidInputError(qtype == ggml_tensor_qtype["asym_int4"],
+                                  "GPTQ / AWQ layers convert to asym_int4 only")
+                is_awq = hasattr(module, "w_bit")
+                has_bias = module.bias is not None and module.bias.abs().sum() != 0
+                device = module.qweight.data.device
+                invalidInputError(device.type != "meta", "converting from meta device is not supported")
+                with _empty_init():
+                    new_linear = LowBitLinear(in_features, out_features, qtype, has_bias, mp_group=mp_group,
+                                              optimize_lm_head=optimize_lm_head, act_order=act_order)
+                weight, g_idx_map = convert_gptq(module, awq=is_awq,
+                                                 llm_awq=is_awq and "LLMAWQ" in str(getattr(module, "backend", "")),
+                                                 act_order=act_order)
+                if act_order:
+                    new_linear.g_idx_map = g_idx_map
+                new_linear._parameters['weight'] = FP4Params(data=weight, requires_grad=False, quantized=True,
+                                                             _shape=(out_features, in_features),
+                                                             convert_shape_only=convert_shape_only,
+                                                             qtype=qtype).to(device)
+                if has_bias:
+                    new_linear._parameters['bias'] = nn.Parameter(module.bias.data).to(device)
+            elif qtype not in (ggml_tensor_qtype["fp16"], ggml_tensor_qtype["bf16"]):
                 if in_features % 64 != 0:
                     continue   # the kernels need in_features to be a multiple of 64
                 cur_qtype, cur_imatrix = get_cur_qtype_and_imatrix(qtype, full_module_name,
@@ -131,7 +219,8 @@ def _replace_with_low_bit_linear(model, qtype, modules_to_not_convert=None,
                 model._modules[name] = new_linear
                 has_been_replaced = True
                 model._modules[name].requires_grad_(False)
-                module.weight = None
+                if isinstance(module, nn.Linear):
+                    module.weight = None
 
         elif embedding_qtype is not None and type(module) == nn.Embedding:
             # convert.py:726-729 of the reference

@@ -192,3 +192,22 @@ def test_from_pretrained_tiny_llama_and_low_bit_round_trip(tmp_path):
     with torch.no_grad():
         got2 = again.to("cuda")(ids.cuda()).logits.float().cpu()
     assert torch.equal(got, got2)
+
+
+@pytest.mark.parametrize("qname,dtype", [("nf4", torch.bfloat16), ("sym_int4", torch.float16)])
+def test_training_backward_is_grad_out_times_the_dequantized_weight(qname, dtype):
+    """MatMulLowBit.backward (reference: low_bit_linear.py:520-541), the QLoRA gradient path."""
+    qtype = Q[qname]
+    n, k = 96, 256
+    w = weights(7100, (n, k))
+    layer = _layer(w, qtype).to("cuda").train()
+    x = torch.randn(2, 5, k).to(dtype).cuda().requires_grad_(True)
+    y = layer(x)
+    assert y.requires_grad and y.shape == (2, 5, n)
+    go = torch.randn_like(y)
+    y.backward(go)
+    wd = torch.from_numpy(orc.dequantize(orc.quantize(w, qtype), qtype, (n, k))).to(dtype).cuda()
+    want = (go.float().view(-1, n) @ wd.float()).view(2, 5, k)
+    assert x.grad.shape == x.shape and x.grad.dtype == dtype
+    assert (x.grad.float() - want).abs().max() <= 1e-2 * want.abs().max()
+    assert layer.weight.grad is None
