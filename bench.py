@@ -50,6 +50,10 @@ def main():
                     help="capture q|k|v and gate|up as parallel graph branches instead of one chain")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the serialized [11008 x 4096] GEMV loop the roofline object is measured on")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the prefill GEMM (M=2048 on [11008 x 4096], sym_int4, fp16) and print its rate")
+    ap.add_argument("--quantize-only", action="store_true",
+                    help="run only the block quantizer (fp32 [11008 x 4096] -> sym_int4, tiled) and print its rate")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no sharding, no collectives); --gpus must be 1",
@@ -70,9 +74,34 @@ def main():
     def stream():
         return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
+    if args.quantize_only:
+        n, k = 11008, 4096
+        ws = [torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02 for _ in range(4)]
+        bs = [torch.empty(blob_bytes(n, k), dtype=torch.uint8, device=dev) for _ in range(4)]
+
+        def quant():
+            for w, b in zip(ws, bs):
+                ggml.lowbit_quantize(w.data_ptr(), b.data_ptr(), SYM_INT4, n, k, ggml.LAYOUT_TILED, stream())
+        for _ in range(max(1, args.warmup)):
+            quant()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            quant()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (args.steps * 4)
+        byts = 4 * n * k + blob_bytes(n, k)
+        print(json.dumps({"quantize": {"kernel": "quantize_tiled_kernel<sym_int4> on fp32 [11008 x 4096]",
+                                       "bound": "hbm", "bytes_per_launch": byts, "avg_launch_us": round(us, 2),
+                                       "achieved": round(byts / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                       "frac": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}}))
+        return
+
     # ---- synthetic weights: N(0, 0.02) with 0.1 % outliers at +-0.5, quantized on the GPU
     layers = []
-    for _ in range(N_LAYERS):
+    for _ in range(4 if args.prefill_only else N_LAYERS):
         mods = []
         for name, n, k in LLAMA2_7B:
             w = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
@@ -155,6 +184,29 @@ def main():
 
     xs, ys = make_io(args.m)
 
+    def prefill_leg(m=2048):
+        """One [11008 x 4096] linear at M rows over 8 distinct weights per graph replay."""
+        gu8 = [b for mods in layers for (name, n, k, b) in mods if name in ("gate", "up")][:8]
+        xp = torch.randn((m, 4096), generator=gen, device=dev, dtype=torch.float32).half()
+        yp = torch.empty((m, 11008), dtype=torch.float16, device=dev)
+
+        def prefill():
+            st = stream()
+            for b in gu8:
+                ggml.lowbit_forward(xp.data_ptr(), b.data_ptr(), yp.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED,
+                                    ggml.DT_F16, m, 11008, 4096, st)
+        g4 = capture(prefill)
+        ms4 = time_graph(g4, 10, 10) / len(gu8)           # clocks settle after some tens of launches
+        flop = 2.0 * m * 11008 * 4096
+        return {"kernel": "gemm_mfma_kernel<sym_int4,f16> on [11008 x 4096], M=%d" % m, "bound": "mfma",
+                "flop_per_launch": flop, "ms": round(ms4, 4), "achieved": round(flop / (ms4 * 1e-3) / 1e12, 1),
+                "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(flop / (ms4 * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill_leg()}))
+        return
+
     # ---- roofline leg: the metric's single shape (N=11008, K=4096) as a serialized chain of
     # launches cycling over the 64 distinct gate/up weights (1.6 GB, far beyond the Infinity Cache)
     gu = [b for mods in layers for (name, n, k, b) in mods if name in ("gate", "up")]
@@ -170,7 +222,10 @@ def main():
     us = ms3 * 1e3 / len(gu)
     roofline = {"bound": "hbm", "kernel": "gemv_mfma_kernel<sym_int4,f16> on [11008 x 4096], M=%d" % args.m,
                 "achieved": round(hb / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(hb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(hb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counters of this very loop
+                # (profiles/gemv_sym_int4_f16_N11008_K4096_M1.md); valid for M = 1 only
+                "traffic": 25510035 if args.m == 1 else None,
                 "bytes_per_launch": hb, "avg_launch_us": round(us, 3),
                 "how": "HIP events around graph replays of 64 chained launches over 64 distinct weights"}
     if args.roofline_only:
@@ -262,23 +317,7 @@ def main():
             extra["sweep_fused_gate_up"] = {"ms_per_step": round(ms6, 4), "launches_per_step": 6 * N_LAYERS,
                                             "GB/s": round(sweep_bytes(args.m) / (ms6 * 1e-3) / 1e9, 1)}
             del g6
-        # prefill: one [11008 x 4096] linear at M = 2048
-        m = 2048
-        xp = torch.randn((m, 4096), generator=gen, device=dev, dtype=torch.float32).half()
-        yp = torch.empty((m, 11008), dtype=torch.float16, device=dev)
-
-        def prefill():
-            st = stream()
-            for b in gu[:8]:
-                ggml.lowbit_forward(xp.data_ptr(), b.data_ptr(), yp.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED,
-                                    ggml.DT_F16, 2048, 11008, 4096, st)
-        g4 = capture(prefill)
-        ms4 = time_graph(g4, 10, 10) / 8                  # clocks settle after some tens of launches
-        flop = 2.0 * m * 11008 * 4096
-        extra["prefill_M2048_N11008_K4096"] = {"ms": round(ms4, 4), "TFLOP/s": round(flop / (ms4 * 1e-3) / 1e12, 1),
-                                               "pct_f16_mfma_peak": round(100 * flop / (ms4 * 1e-3) / 1e12 /
-                                                                          MFMA_F16_PEAK_TFLOPS, 2)}
-        del xp, yp, g4
+        extra["prefill_M2048_N11008_K4096"] = prefill_leg(2048)
         extra.update(other_configs(ggml, torch, gen, dev, layers[0], capture, time_graph, stream))
         out["extra"] = extra
 
