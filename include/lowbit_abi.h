@@ -134,6 +134,16 @@ int lowbit_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, v
 int lowbit_mlp_forward(const void *x, const void *w_gate, const void *w_up, void *y, int qtype, int act_dtype,
                        int64_t M, int64_t N, int64_t K, int act, void *stream);
 
+/* xe_linear.moe_forward_vec (python/llm/src/ipex_llm/transformers/models/deepseek.py:290-315): one
+ * token through its top_k experts without the host reading the routing result.
+ * y[hidden] = sum_j topk_weight[j] * down[e_j](act(gate[e_j] x) .* up[e_j] x), e_j = topk_ids[j].
+ * topk_ids (int32, clamped to [0, n_experts)), topk_weight (fp32) and the three pointer tables (one tiled weight per expert,
+ * gate / up [inter, hidden], down [hidden, inter]) live in DEVICE memory; workspace is caller-owned
+ * device memory of top_k * inter activations (16-byte aligned).  Two launches on `stream`. */
+int lowbit_moe_forward(const void *x, const int32_t *topk_ids, const float *topk_weight, int top_k, int n_experts,
+                       const void *const *gates, const void *const *ups, const void *const *downs, void *workspace,
+                       void *y, int qtype, int act_dtype, int64_t hidden, int64_t inter, int act, void *stream);
+
 /* Grouped product for mixture-of-experts layers, one launch for all experts.  The reference has
  * no single call for it: it loops over the experts in Python and calls each expert's LowBitLinear
  * on the rows routed to it (python/llm/src/ipex_llm/transformers/models/qwen2_moe.py:375-430 is the

@@ -11,6 +11,9 @@ int launch_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, v
                            int64_t K, int layout, int out_dtype, hipStream_t st);
 int launch_mlp_gemv(const void *x, const void *wg, const void *wu, void *y, int qtype, int act_dtype, int M, int N,
                     int K, int act, hipStream_t st);
+int launch_moe_gemv(const void *x, const int32_t *ids, const float *route_w, int slots, int n_exp, const void *gates,
+                    const void *ups, const void *downs, void *h, void *y, int qtype, int act_dtype, int hidden,
+                    int inter, int act, hipStream_t st);
 int launch_quantize(const float *src, void *dst, int qtype, int64_t N, int64_t K, int layout, hipStream_t st);
 int launch_relayout(const void *src, void *dst, int qtype, int64_t N, int64_t K, int src_layout, hipStream_t st);
 int launch_dequantize(const void *w, void *out, int qtype, int64_t N, int64_t K, int layout, int out_dtype,
@@ -174,6 +177,26 @@ int lowbit_mlp_forward(const void *x, const void *w_gate, const void *w_up, void
     if (!w_up || !aligned16(w_up)) return fail(LOWBIT_EARG, "lowbit_mlp_forward: null or misaligned pointer");
     return check_launch(launch_mlp_gemv(x, w_gate, w_up, y, qtype, act_dtype, (int)M, (int)N, (int)K, act,
                                         (hipStream_t)stream), "lowbit_mlp_forward");
+}
+
+int lowbit_moe_forward(const void *x, const int32_t *topk_ids, const float *topk_weight, int top_k, int n_experts,
+                       const void *const *gates, const void *const *ups, const void *const *downs, void *workspace,
+                       void *y, int qtype, int act_dtype, int64_t hidden, int64_t inter, int act, void *stream) {
+    if (int rc = check_weight_shape("lowbit_moe_forward", qtype, inter, hidden, LOWBIT_LAYOUT_TILED)) return rc;
+    if (int rc = check_weight_shape("lowbit_moe_forward", qtype, hidden, inter, LOWBIT_LAYOUT_TILED)) return rc;
+    if (act_dtype != LOWBIT_DT_F16 && act_dtype != LOWBIT_DT_BF16)
+        return fail(LOWBIT_EDTYPE, "lowbit_moe_forward: activations must be f16 or bf16");
+    if (act != LOWBIT_ACT_SILU && act != LOWBIT_ACT_GELU)
+        return fail(LOWBIT_EARG, "lowbit_moe_forward: activation must be LOWBIT_ACT_SILU or LOWBIT_ACT_GELU");
+    if (top_k < 1 || top_k > 64 || top_k * inter > 0x7fffffff || n_experts < 1)
+        return fail(LOWBIT_ESIZE, "lowbit_moe_forward: top_k must be 1 .. 64 and n_experts positive");
+    if (hidden == 0 || inter == 0) return 0;
+    if (!x || !topk_ids || !topk_weight || !gates || !ups || !downs || !workspace || !y || !aligned16(x) ||
+        !aligned16(workspace))
+        return fail(LOWBIT_EARG, "lowbit_moe_forward: null or misaligned pointer");
+    return check_launch(launch_moe_gemv(x, topk_ids, topk_weight, top_k, n_experts, gates, ups, downs, workspace, y, qtype,
+                                        act_dtype, (int)hidden, (int)inter, act, (hipStream_t)stream),
+                        "lowbit_moe_forward");
 }
 
 int lowbit_grouped_forward(const void *x, const void *const *w, void *y, const int32_t *group_offsets, int n_groups,

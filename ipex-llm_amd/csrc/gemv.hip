@@ -159,10 +159,20 @@ constexpr int GEMV_LDS_X_BUDGET = 64 * 1024;
 // DUAL: the fused gate/up projection of a gated MLP (xe_linear.mlp_forward_xpu,
 // python/llm/src/ipex_llm/transformers/models/common.py:145-158): the workgroup walks the same
 // tile row of two weights with one copy of x and writes act(x Wg^T) * (x Wu^T).
-template <int QT, typename AT, int MT, int U, int XN, bool DUAL>
+//
+// MOE: the two launches of a fused mixture-of-experts decode step (xe_linear.moe_forward_vec,
+// python/llm/src/ipex_llm/transformers/models/deepseek.py:290-315).  w / w2 are then tables of
+// weight pointers in device memory and ids[j] names the expert of routing slot j, so that the host
+// never has to read the routing result.
+//   MOE == 1 (with DUAL): blockIdx.y = slot j; row j of y = act(x Wg[e]^T) * (x Wu[e]^T).
+//   MOE == 2: x is the [slots, K / slots] output of the first launch, read as one long vector;
+//             tile g of the K walk belongs to slot g / ge and is scaled by route_w[slot]:
+//             y = sum_j route_w[j] * (x_j Wd[e_j]^T).
+template <int QT, typename AT, int MT, int U, int XN, bool DUAL, int MOE>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                          const uint8_t *__restrict__ w2, AT *__restrict__ y, int M,
-                                                         int N, int K, int act) {
+                                                         int N, int K, int act, const int32_t *__restrict__ ids,
+                                                         const float *__restrict__ route_w, int ge, int n_exp) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
     constexpr bool IS4 = (F::BITS == 4);
@@ -189,11 +199,27 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     // they may hold anything: they re-read a valid row, which LDS serves as a broadcast.
     int m_of_r = (r >> 2) * MT + ((r & 3) < MT ? (r & 3) : MT - 1);
     m_of_r = m_of_r < M ? m_of_r : M - 1;
-    const uint8_t *wrow = w + (int64_t)blockIdx.x * G * F::TILE_BYTES;
+    gbytes wrow = nullptr, wrow2 = nullptr;
+    if constexpr (MOE == 0) {
+        wrow = (gbytes)w + (int64_t)blockIdx.x * G * F::TILE_BYTES;
+        if constexpr (DUAL) wrow2 = (gbytes)w2 + (int64_t)blockIdx.x * G * F::TILE_BYTES;
+    } else if constexpr (MOE == 1) {
+        // ids come from device memory: clamp, so that a bad id cannot send a load astray
+        const int e = min(max(ids[blockIdx.y], 0), n_exp - 1);
+        wrow = (gbytes)((const uint8_t *const *)w)[e] + (int64_t)blockIdx.x * G * F::TILE_BYTES;
+        wrow2 = (gbytes)((const uint8_t *const *)w2)[e] + (int64_t)blockIdx.x * G * F::TILE_BYTES;
+        y += (int64_t)blockIdx.y * N;
+    }
+    // MOE == 2: tile g -> slot g / ge; its weight row starts at table[ids[slot]] + blockIdx.x * ge tiles
+    auto moe_tile = [&](int g, float &rw) -> gbytes {
+        const int slot = g / ge;
+        rw = route_w[slot];
+        return (gbytes)((const uint8_t *const *)w)[min(max(ids[slot], 0), n_exp - 1)] +
+               ((int64_t)blockIdx.x * ge + (g - slot * ge)) * F::TILE_BYTES;
+    };
     AT *xs = (AT *)smem + (int64_t)wave * (XN * 512);       // [XN*64/(SLICE/8)][SLICE], private to this wave
     const AT *xa = xs + m_of_r * SLICE + 8 * c;
 
-    const uint8_t *wrow2 = DUAL ? w2 + (int64_t)blockIdx.x * G * F::TILE_BYTES : nullptr;
     float acc[NW * MT];
 #pragma unroll
     for (int i = 0; i < NW * MT; i++) acc[i] = 0.0f;
@@ -220,10 +246,13 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
         }
         __builtin_amdgcn_sched_barrier(0);                  // keep the x loads ahead of the weight loads
         TileRegs<QT> tr[NW * U];
+        float rw[U];
 #pragma unroll
         for (int t = 0; t < U; t++) {
-            const int g = gw + t;
-            load_tile<QT>(wrow + (int64_t)(g < G ? g : G - 1) * F::TILE_BYTES, lane, r, tr[t]);
+            const int g = gw + t < G ? gw + t : G - 1;
+            rw[t] = 1.0f;
+            if constexpr (MOE == 2) load_tile<QT>(moe_tile(g, rw[t]), lane, r, tr[t]);
+            else load_tile<QT>(wrow + (int64_t)g * F::TILE_BYTES, lane, r, tr[t]);
         }
         if constexpr (DUAL) {
 #pragma unroll
@@ -260,6 +289,10 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
                     else b = Unpack8<QT, AT>::run(tl.q1[2 * (j - 2)], tl.q1[2 * (j - 2) + 1]);
                     float d, mn;
                     tile_scale<QT>(tl, j, d, mn);
+                    if constexpr (MOE == 2) {
+                        d *= rw[t];
+                        mn *= rw[t];
+                    }
                     d = live ? d : 0.0f;
                     mn = live ? mn : 0.0f;
                     const f32x4 p = mfma16(a[j], b, zero4);
@@ -338,9 +371,10 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const AT *__restrict_
 
 // -------------------------------------------------------------- launch
 
-template <int QT, typename AT, int MT, int U, int XN, bool DUAL = false>
+template <int QT, typename AT, int MT, int U, int XN, bool DUAL = false, int MOE = 0>
 static void launch_mfma(const AT *x, const uint8_t *w, AT *y, int M, int N, int K, int waves, hipStream_t st,
-                        const uint8_t *w2 = nullptr, int act = 0) {
+                        const uint8_t *w2 = nullptr, int act = 0, const int32_t *ids = nullptr,
+                        const float *route_w = nullptr, int ge = 0, int slots = 1, int n_exp = 1) {
     const int G = K / TILE_COLS;
     // waves: enough that one round covers K, within the block size limit and the LDS budget for x
     int wv = (G + U - 1) / U;
@@ -350,8 +384,8 @@ static void launch_mfma(const AT *x, const uint8_t *w, AT *y, int M, int N, int 
     if (waves > 0 && waves < wv) wv = waves;
     if (wv < 1) wv = 1;
     const size_t lds = (size_t)wv * XN * 512 * sizeof(AT);
-    hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, MT, U, XN, DUAL>), dim3(N / TILE_ROWS), dim3(64 * wv), lds, st, x, w, w2,
-                       y, M, N, K, act);
+    hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, MT, U, XN, DUAL, MOE>), dim3(N / TILE_ROWS, MOE == 1 ? slots : 1),
+                       dim3(64 * wv), lds, st, x, w, w2, y, M, N, K, act, ids, route_w, ge, n_exp);
 }
 
 template <int QT, typename AT>
@@ -428,6 +462,40 @@ int launch_mlp_gemv(const void *x, const void *wg, const void *wu, void *y, int 
     case QT_SYM_INT8: return launch_mlp_q<QT_SYM_INT8>(x, wg, wu, y, act_dtype, M, N, K, act, st);
     case QT_NF4: return launch_mlp_q<QT_NF4>(x, wg, wu, y, act_dtype, M, N, K, act, st);
     case QT_FP8_E4M3: return launch_mlp_q<QT_FP8_E4M3>(x, wg, wu, y, act_dtype, M, N, K, act, st);
+    default: return -2;
+    }
+}
+
+template <int QT, typename AT>
+static int launch_moe_t(const void *x, const int32_t *ids, const float *route_w, int slots, int n_exp, const void *gates,
+                        const void *ups, const void *downs, void *h, void *y, int hidden, int inter, int act,
+                        hipStream_t st) {
+    // h[slots, inter] = act(x Wg[e]^T) * (x Wu[e]^T), then y[hidden] = sum_j route_w[j] * h[j] Wd[e_j]^T
+    launch_mfma<QT, AT, 1, 4, 1, true, 1>((const AT *)x, (const uint8_t *)gates, (AT *)h, 1, inter, hidden, 0, st,
+                                          (const uint8_t *)ups, act, ids, nullptr, 0, slots, n_exp);
+    launch_mfma<QT, AT, 1, 4, 1, false, 2>((const AT *)h, (const uint8_t *)downs, (AT *)y, 1, hidden, slots * inter, 0,
+                                           st, nullptr, 0, ids, route_w, inter / TILE_COLS, slots, n_exp);
+    return 0;
+}
+
+template <int QT>
+static int launch_moe_q(const void *x, const int32_t *ids, const float *route_w, int slots, int n_exp, const void *gates,
+                        const void *ups, const void *downs, void *h, void *y, int dt, int hidden, int inter, int act,
+                        hipStream_t st) {
+    if (dt == DT_F16) return launch_moe_t<QT, _Float16>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, hidden, inter, act, st);
+    if (dt == DT_BF16) return launch_moe_t<QT, __bf16>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, hidden, inter, act, st);
+    return -4;
+}
+
+int launch_moe_gemv(const void *x, const int32_t *ids, const float *route_w, int slots, int n_exp, const void *gates,
+                    const void *ups, const void *downs, void *h, void *y, int qtype, int act_dtype, int hidden,
+                    int inter, int act, hipStream_t st) {
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_moe_q<QT_SYM_INT4>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, act_dtype, hidden, inter, act, st);
+    case QT_ASYM_INT4: return launch_moe_q<QT_ASYM_INT4>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, act_dtype, hidden, inter, act, st);
+    case QT_SYM_INT8: return launch_moe_q<QT_SYM_INT8>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, act_dtype, hidden, inter, act, st);
+    case QT_NF4: return launch_moe_q<QT_NF4>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, act_dtype, hidden, inter, act, st);
+    case QT_FP8_E4M3: return launch_moe_q<QT_FP8_E4M3>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, act_dtype, hidden, inter, act, st);
     default: return -2;
     }
 }

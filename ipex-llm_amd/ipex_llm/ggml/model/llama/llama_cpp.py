@@ -194,6 +194,17 @@ _lib.lowbit_mlp_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_in
 _lib.lowbit_mlp_forward.restype = c_int
 
 
+_lib.lowbit_moe_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                    c_void_p, c_int, c_int, c_int64, c_int64, c_int, c_void_p]
+_lib.lowbit_moe_forward.restype = c_int
+
+
+def lowbit_moe_forward(x, topk_ids, topk_weight, top_k, n_experts, gates, ups, downs, workspace, y, qtype, act_dtype,
+                       hidden, inter, act, stream):
+    _check(_lib.lowbit_moe_forward(x, topk_ids, topk_weight, top_k, n_experts, gates, ups, downs, workspace, y, qtype,
+                                   act_dtype, hidden, inter, act, stream), "lowbit_moe_forward")
+
+
 def lowbit_dequantize_rows(w, rows, n_rows, dst, qtype, n, k, layout, out_dtype, stream):
     _check(_lib.lowbit_dequantize_rows(w, rows, n_rows, dst, qtype, n, k, layout, out_dtype, stream),
            "lowbit_dequantize_rows")

@@ -59,6 +59,30 @@ def grouped_forward(x_sorted: torch.Tensor, group_offsets: torch.Tensor, experts
     return y
 
 
+def moe_forward_vec(x: torch.Tensor, topk_ids: torch.Tensor, topk_weight: torch.Tensor, gates: ExpertWeights,
+                    ups: ExpertWeights, downs: ExpertWeights, act: int = 0):
+    """xe_linear.moe_forward_vec (models/deepseek.py:290-315 of the reference): one token through its top-k
+    experts in two launches.  Nothing is read back to the host: the expert ids stay on the GPU.
+    x [1, hidden]; topk_ids / topk_weight [1, top_k]; returns [1, hidden]."""
+    hidden, inter = gates.in_len, gates.out_len
+    invalidInputError(x.dim() == 2 and x.shape == (1, hidden) and x.dtype in (torch.float16, torch.bfloat16),
+                      "moe_forward_vec expects one fp16 / bf16 row of x")
+    invalidInputError((ups.qtype, ups.out_len, ups.in_len) == (gates.qtype, inter, hidden)
+                      and (downs.qtype, downs.out_len, downs.in_len) == (gates.qtype, hidden, inter),
+                      "gate / up / down experts do not fit together")
+    top_k = topk_ids.numel()
+    ids = topk_ids.reshape(-1).to(torch.int32)
+    rw = topk_weight.reshape(-1).to(torch.float32)
+    xc = x.contiguous()
+    work = torch.empty((top_k, inter), dtype=x.dtype, device=x.device)
+    y = torch.empty((1, hidden), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        ggml.lowbit_moe_forward(xc.data_ptr(), ids.data_ptr(), rw.data_ptr(), top_k, len(gates.blobs),
+                                gates.ptrs.data_ptr(), ups.ptrs.data_ptr(), downs.ptrs.data_ptr(), work.data_ptr(),
+                                y.data_ptr(), gates.qtype, _DT[x.dtype], hidden, inter, act, _stream())
+    return y
+
+
 def moe_ffn_reference(hidden, router_logits, w1, w3, w2, top_k=2):
     """The per-expert loop: w1/w3/w2 are lists of LowBitLinear (gate, up, down)."""
     weights, experts = route_top_k(router_logits, top_k)

@@ -62,3 +62,32 @@ def test_moe_ffn_grouped_equals_per_expert_loop(qname, dtype):
     ref = moe_ffn_reference(x, logits, w1, w3, w2).float()
     got = moe_ffn_grouped(x, logits, ExpertWeights(w1), ExpertWeights(w3), ExpertWeights(w2)).float()
     assert (got - ref).abs().max() <= 1e-2 * ref.abs().max()
+
+
+@pytest.mark.parametrize("qname,dtype", [("sym_int4", torch.float16), ("fp8_e4m3", torch.bfloat16),
+                                         ("nf4", torch.bfloat16)])
+def test_moe_forward_vec_equals_the_per_expert_decode_loop(qname, dtype):
+    from ipex_llm.transformers.moe import moe_forward_vec
+    qtype = Q[qname]
+    n_exp, hidden, ffn, top_k = 6, 256, 640, 3         # 5 tiles per expert: slots straddle a wave's tiles
+    w1, r1 = _experts(n_exp, ffn, hidden, qtype, 8400)
+    w3, r3 = _experts(n_exp, ffn, hidden, qtype, 8500)
+    w2, r2 = _experts(n_exp, hidden, ffn, qtype, 8600)
+    torch.manual_seed(4)
+    x = torch.randn(1, hidden).to(dtype).cuda()
+    ids = torch.tensor([[4, 0, 5]], device="cuda")
+    wts = torch.tensor([[0.5, 0.3, 0.2]], device="cuda")
+    got = moe_forward_vec(x, ids, wts, ExpertWeights(w1), ExpertWeights(w3), ExpertWeights(w2)).float().cpu().numpy()
+    # the loop of the reference (models/deepseek.py:317-327), in exact arithmetic on the oracle's weights
+    xf = x.float().cpu().numpy()
+    want = np.zeros((1, hidden), dtype=np.float64)
+    for e, wt in zip(ids[0].tolist(), wts[0].tolist()):
+        g = orc.mul_mat_exact(orc.quantize(r1[e], qtype), xf, (ffn, hidden), qtype).astype(np.float64)
+        u = orc.mul_mat_exact(orc.quantize(r3[e], qtype), xf, (ffn, hidden), qtype).astype(np.float64)
+        h = (g / (1.0 + np.exp(-g)) * u).astype(np.float32)
+        want += wt * orc.mul_mat_exact(orc.quantize(r2[e], qtype), h, (hidden, ffn), qtype)
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max()
+    # and against the modules themselves
+    loop = sum(wt * w2[e](torch.nn.functional.silu(w1[e](x)) * w3[e](x)).float()
+               for e, wt in zip(ids[0].tolist(), wts[0].tolist())).cpu().numpy()
+    assert np.abs(got - loop).max() <= 1e-2 * np.abs(loop).max()
