@@ -164,6 +164,15 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // so the GEMM is built on it.  The accumulator is pinned to accumulation registers, in place,
 // through inline assembly: left to the compiler, the 128 accumulators migrate between register
 // ranges across the unrolled K steps and get copied back every iteration.
+// Waits for every outstanding global load, the LDS-DMA ones included.  Spelled with the builtin
+// (s_waitcnt vmcnt(0), other counters untouched) so that the compiler's own wait-count bookkeeping
+// sees it: after an opaque inline-asm wait it would still believe the weight loads of the previous
+// step to be in flight and wait for them again - in fact for the LDS-DMA loads just issued.
+__device__ inline void wait_all_loads() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
+}
+
 __device__ inline void mfma_acc(f32x16 &c, f16x8 a, f16x8 b) {
     asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
@@ -420,18 +429,18 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             WRegs w0, w1;
             dma_x(0, xs0);
             load_w(0, w0);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            wait_all_loads();
             __syncthreads();
             for (int kt = 0; kt + 1 < G; kt += 2) {
                 dma_x(kt + 1, xs1);
                 load_w(kt + 1, w1);
                 compute(xs0, w0, mbc);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                wait_all_loads();
                 __syncthreads();
                 dma_x(kt + 2, xs0);                          // past the end: a clamped, unused re-read
                 load_w(kt + 2, w0);
                 compute(xs1, w1, mbc);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                wait_all_loads();
                 __syncthreads();
             }
             if (G & 1) compute(xs0, w0, mbc);
