@@ -13,7 +13,8 @@ than the overlap gains).  Weights (3.64 GB) are resident
 in HBM before the timed region and exceed the 256 MB Infinity Cache, so every
 sweep streams them from HBM.
 
-Prints ONE JSON line (see README / DESIGN.md for the fields).
+Prints ONE JSON line: metric / value / unit, the roofline and cpu_baseline objects, and one timed leg per
+other configuration under "extra".
 """
 import argparse
 import ctypes
