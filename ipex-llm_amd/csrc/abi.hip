@@ -61,7 +61,7 @@ static int check_weight_shape(const char *what, int qtype, int64_t N, int64_t K,
     if (K % qk) return fail(LOWBIT_ESHAPE, "%s: K=%lld is not a multiple of the block size %d", what, (long long)K, qk);
     if (layout != LOWBIT_LAYOUT_GGML && layout != LOWBIT_LAYOUT_TILED)
         return fail(LOWBIT_EARG, "%s: unknown layout %d", what, layout);
-    if (layout == LOWBIT_LAYOUT_TILED && !lowbit_tileable(qtype, N, K))
+    if (layout == LOWBIT_LAYOUT_TILED && N * K != 0 && !lowbit_tileable(qtype, N, K))   // empty: nothing to lay out
         return fail(LOWBIT_ESHAPE, "%s: [%lld, %lld] needs N %% 16 == 0 and K %% 128 == 0 for the tiled layout", what,
                     (long long)N, (long long)K);
     if (N > 0x7fffffff || K > 0x7fffffff) return fail(LOWBIT_ESIZE, "%s: dimension exceeds 2^31", what);

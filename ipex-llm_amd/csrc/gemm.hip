@@ -390,9 +390,14 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
 
     auto epilogue = [&](auto mbc_) {
         constexpr int MBC = decltype(mbc_)::value;
-    // the MFMAs above are opaque to the compiler's hazard tracking: give the last results time
-    // to land before the accumulation registers are read back
-    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7");
+    // The MFMAs above are opaque to the compiler's hazard tracking: give the last results time to
+    // land before the accumulation registers are read back (a 16-pass MFMA needs 18 wait states
+    // before its result may be read; 64 are spent).  The accumulators are operands of the statement,
+    // so that no read of them can be scheduled ahead of it.
+#pragma unroll
+    for (int mb = 0; mb < MBC; mb++)
+        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7"
+                     : "+a"(acc[mb][0]), "+a"(acc[mb][1]));
     // C layout of the 32x32 block: lane = 32*g + col (col = x row within the block), register i =
     // weight row 8*(i/4) + 4*g + i%4: four consecutive n per group of registers
 #pragma unroll

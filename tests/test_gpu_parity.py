@@ -3,9 +3,10 @@ import numpy as np
 import pytest
 import torch
 
+import ipex_llm.ggml.model.llama.llama_cpp as ggml
 import lowbit_oracle as orc
-from gpu_util import (ALL, FP8, NF4, Q4_0, Q4_1, Q8_0, acts, dev_dequantize, dev_matmul, dev_quantize,
-                      dev_relayout, weights)
+from gpu_util import (ALL, DT, FP8, NF4, Q4_0, Q4_1, Q8_0, acts, dev_dequantize, dev_matmul, dev_quantize,
+                      dev_relayout, stream, weights)
 
 pytestmark = pytest.mark.gpu
 
@@ -202,3 +203,76 @@ def test_gemm_prefill_shape_sym_and_asym_int4():
         wd = orc.dequantize(blob_np, qtype, (n, k)).astype(np.float64)
         y_exact = x.float().numpy()[rows].astype(np.float64) @ wd.T
         assert np.abs(y[rows] - y_exact).max() <= 2e-3 * np.abs(y_exact).max()
+
+
+@pytest.mark.parametrize("qtype,dtype", [(Q4_0, torch.float16), (Q4_1, torch.bfloat16), (Q8_0, torch.float16),
+                                         (NF4, torch.bfloat16), (FP8, torch.bfloat16)])
+def test_gemm_with_more_tiles_than_cus_against_oracle(qtype, dtype):
+    # 10 x 28 = 280 tiles of 128 x 256: the form of the GEMM with two workgroups per CU; M leaves a tail
+    # tile of 48 rows (two 32-row blocks), K = 384 is an odd number of 128-column steps
+    m, n, k = 1200, 7168, 384
+    w = weights(5300 + qtype, (n, k))
+    x = acts(5301, m, k, dtype)
+    blob_np = orc.quantize(w, qtype)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n, fn="gemm")
+    y_exact = orc.mul_mat_exact(blob_np, x.float().numpy(), (n, k), qtype)
+    assert np.isfinite(y).all()
+    tol = 2e-3 if dtype == torch.float16 else 8e-3
+    assert np.abs(y - y_exact).max() <= tol * np.abs(y_exact).max()
+
+
+def test_gemm_tail_tile_of_at_most_32_rows():
+    m, n, k = 1040, 7168, 256            # 8 full row tiles + one of 16 rows: the one-block copy of the loop
+    w = weights(5310, (n, k))
+    x = acts(5311, m, k, torch.float16)
+    blob = dev_quantize(w, Q4_0, TILED)
+    y = dev_matmul(x, blob, Q4_0, TILED, n, fn="gemm")
+    y_exact = orc.mul_mat_exact(orc.quantize(w, Q4_0), x.float().numpy(), (n, k), Q4_0)
+    assert np.abs(y - y_exact).max() <= 2e-3 * np.abs(y_exact).max()
+
+
+def test_full_size_prefill_agrees_with_the_decode_kernel_and_is_linear():
+    """BASELINE configs[2] at full size ([11008 x 4096], M = 2048), where the oracle would take
+    minutes: the GEMM must agree with the (oracle-checked) GEMV on sampled rows, and be linear in x."""
+    n, k, m = 11008, 4096, 2048
+    w = weights(5320, (n, k))
+    blob = dev_quantize(w, Q4_0, TILED)
+    x = acts(5321, m, k, torch.float16)
+    y = dev_matmul(x, blob, Q4_0, TILED, n, fn="gemm")
+    rows = [0, 1, 127, 128, 1000, 2047]
+    yv = dev_matmul(x[rows], blob, Q4_0, TILED, n, fn="gemv")
+    assert np.abs(y[rows] - yv).max() <= 2e-3 * np.abs(yv).max()
+    # power-of-two scalings and the sign of x commute with the product up to rounding: the MFMA's
+    # internal fp32 accumulation is not sign-symmetric (seen as ~1e-7 differences where the sum cancels
+    # to almost nothing), so allow that plus the final fp16 rounding step
+    slack = 2 * np.maximum(np.abs(y) * 2.0 ** -10, 2.0 ** -24) + 1e-6 * np.abs(y).max()
+    y2 = dev_matmul(x * 2, blob, Q4_0, TILED, n, fn="gemm")
+    assert (np.abs(y2 - 2 * y) <= 2 * slack).all() and (y2 == 2 * y).mean() > 0.999
+    yn = dev_matmul(-x, blob, Q4_0, TILED, n, fn="gemm")
+    assert (np.abs(yn + y) <= slack).all() and (yn == -y).mean() > 0.999
+    # a row of the oracle for good measure
+    want = orc.mul_mat_exact(orc.quantize(w, Q4_0), x[5:6].float().numpy(), (n, k), Q4_0)
+    assert np.abs(y[5:6] - want).max() <= 2e-3 * np.abs(want).max()
+
+
+def test_device_entry_points_reject_bad_arguments():
+    blob = dev_quantize(weights(5330, (32, 256)), Q4_0, TILED)
+    x = acts(5331, 2, 256, torch.float16).cuda()
+    y = torch.empty((2, 32), dtype=torch.float16, device="cuda")
+    ok = (x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 2, 32, 256)
+    ggml.lowbit_forward(*ok, stream())
+    bad = {"qtype": (3, 99), "layout": (4, 7), "dtype": (5, 2), "M": (6, -1), "K": (8, 250), "x": (0, 0),
+           "x alignment": (0, x.data_ptr() + 2)}
+    for what, (pos, val) in bad.items():
+        args = list(ok)
+        args[pos] = val
+        with pytest.raises(RuntimeError):
+            ggml.lowbit_forward(*args, stream())
+    with pytest.raises(RuntimeError, match="tiled"):           # 24 rows cannot be tiled
+        ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 2, 24, 256,
+                            stream())
+    # empty problems are no-ops
+    ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 0, 32, 256, stream())
+    ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 2, 0, 256, stream())
+    torch.cuda.synchronize()
