@@ -276,3 +276,15 @@ def test_device_entry_points_reject_bad_arguments():
     ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 0, 32, 256, stream())
     ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 2, 0, 256, stream())
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("qtype,n,k", [(NF4, 8192, 28672), (Q8_0, 28672, 8192), (NF4, 1024, 8192)])
+@pytest.mark.parametrize("m", [1, 16])
+def test_llama3_70b_shapes_decode_against_oracle(qtype, n, k, m):
+    # BASELINE configs[3] at full size (bf16 activations); long K runs several rounds of the K walk
+    w = weights(5400 + qtype, (n, k), std=0.015, outliers=False)
+    x = acts(5401 + m, m, k, torch.bfloat16)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n)
+    y_exact = orc.mul_mat_exact(orc.quantize(w, qtype), x.float().numpy(), (n, k), qtype)
+    assert np.abs(y - y_exact).max() <= 8e-3 * np.abs(y_exact).max()

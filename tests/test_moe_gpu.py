@@ -29,9 +29,10 @@ def _experts(n_exp, n, k, qtype, seed):
                                          ("nf4", torch.bfloat16), ("sym_int8", torch.float16)])
 def test_grouped_forward_matches_oracle_per_group(qname, dtype):
     qtype = Q[qname]
-    n_exp, n, k = 5, 272, 256
+    n_exp, n, k = 8, 272, 384                          # 3 steps of 128 columns: an odd count
     lins, raw = _experts(n_exp, n, k, qtype, 8000)
-    counts = [130, 0, 1, 17, 129]                      # empty group, single row, partial and full tiles
+    # empty group, single row, tiles of 1 / 2 / 3 / 4 row blocks, a full tile plus one row
+    counts = [130, 0, 1, 17, 129, 40, 64, 97]
     rows = sum(counts)
     torch.manual_seed(1)
     x = torch.randn(rows, k).to(dtype).cuda()
