@@ -28,29 +28,29 @@ template <int QT, typename AT> struct Unpack;
 // 4-bit integer codes, fp16: 0x6400 | q is the half 1024 + q; 0x6400 | q << 4 is 1024 + 16 q.
 template <> struct Unpack<QT_SYM_INT4, _Float16> {
     static constexpr float OFFSET = 0.0f;
-    __device__ static f16x8 run(uint32_t v, const void *) {
+    __device__ static f16x8 run(uint32_t v, const void *, uint32_t magic) {
         const f16x2 k1032 = {(_Float16)1032.0f, (_Float16)1032.0f};
         const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
         const f16x2 k72 = {(_Float16)72.0f, (_Float16)72.0f};
         const uint32_t v8 = v >> 8;
-        f16x2 t0 = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1032;
-        f16x2 t1 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k72);
-        f16x2 t2 = __builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, 0x64006400u)) - k1032;
-        f16x2 t3 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, 0x64006400u)), k16th, -k72);
+        f16x2 t0 = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, magic)) - k1032;
+        f16x2 t1 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, magic)), k16th, -k72);
+        f16x2 t2 = __builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, magic)) - k1032;
+        f16x2 t3 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, magic)), k16th, -k72);
         return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
     }
 };
 template <> struct Unpack<QT_ASYM_INT4, _Float16> {
     static constexpr float OFFSET = 0.0f;
-    __device__ static f16x8 run(uint32_t v, const void *) {
+    __device__ static f16x8 run(uint32_t v, const void *, uint32_t magic) {
         const f16x2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
         const f16x2 k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
         const f16x2 k64 = {(_Float16)64.0f, (_Float16)64.0f};
         const uint32_t v8 = v >> 8;
-        f16x2 t0 = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, 0x64006400u)) - k1024;
-        f16x2 t1 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, 0x64006400u)), k16th, -k64);
-        f16x2 t2 = __builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, 0x64006400u)) - k1024;
-        f16x2 t3 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, 0x64006400u)), k16th, -k64);
+        f16x2 t0 = __builtin_bit_cast(f16x2, and_or(v, 0x000f000fu, magic)) - k1024;
+        f16x2 t1 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v, 0x00f000f0u, magic)), k16th, -k64);
+        f16x2 t2 = __builtin_bit_cast(f16x2, and_or(v8, 0x000f000fu, magic)) - k1024;
+        f16x2 t3 = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, and_or(v8, 0x00f000f0u, magic)), k16th, -k64);
         return f16x8{t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
     }
 };
@@ -58,12 +58,12 @@ template <> struct Unpack<QT_ASYM_INT4, _Float16> {
 // afterwards through the row sum of x, which a second MFMA against all-ones provides.
 template <int QT> struct UnpackInt4Bf16 {
     static constexpr float OFFSET = (QT == QT_SYM_INT4) ? 136.0f : 128.0f;
-    __device__ static bf16x8 run(uint32_t v, const void *) {
+    __device__ static bf16x8 run(uint32_t v, const void *, uint32_t magic) {
         u32x4 t;
-        t[0] = and_or(v, 0x000f000fu, 0x43004300u);
-        t[1] = and_or(v >> 4, 0x000f000fu, 0x43004300u);
-        t[2] = and_or(v >> 8, 0x000f000fu, 0x43004300u);
-        t[3] = and_or(v >> 12, 0x000f000fu, 0x43004300u);
+        t[0] = and_or(v, 0x000f000fu, magic);
+        t[1] = and_or(v >> 4, 0x000f000fu, magic);
+        t[2] = and_or(v >> 8, 0x000f000fu, magic);
+        t[3] = and_or(v >> 12, 0x000f000fu, magic);
         return __builtin_bit_cast(bf16x8, t);
     }
 };
@@ -73,7 +73,7 @@ template <> struct Unpack<QT_ASYM_INT4, __bf16> : UnpackInt4Bf16<QT_ASYM_INT4> {
 // nf4: code-book lookup from a 16-entry table in LDS (entries already in the activation type).
 template <typename AT> struct Unpack<QT_NF4, AT> {
     static constexpr float OFFSET = 0.0f;
-    __device__ static typename Vec8<AT>::type run(uint32_t v, const void *lut_) {
+    __device__ static typename Vec8<AT>::type run(uint32_t v, const void *lut_, uint32_t) {
         const AT *lut = (const AT *)lut_;
         typename Vec8<AT>::type r;
         r[0] = lut[v & 0xf]; r[2] = lut[(v >> 4) & 0xf]; r[4] = lut[(v >> 8) & 0xf]; r[6] = lut[(v >> 12) & 0xf];
@@ -228,6 +228,12 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     for (int i = 0; i < NW * MT; i++) acc[i] = 0.0f;
     const V8 ones = ones8<AT>();
     const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    // exponent pattern OR-ed onto 4-bit codes (fp16 1024, bf16 128), held in a vector register: as a
+    // literal it would share the instruction's one constant slot with the nibble mask and split every
+    // v_and_or_b32 into an AND and an OR
+    uint32_t magic;
+    if constexpr (sizeof(AT) == 2 && __is_same(AT, _Float16)) asm("v_mov_b32 %0, 0x64006400" : "=v"(magic));
+    else asm("v_mov_b32 %0, 0x43004300" : "=v"(magic));
 
     for (int g0 = 0; g0 < G; g0 += W * U) {
         const int gw = g0 + wave * U;
@@ -294,7 +300,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     V8 b;
-                    if constexpr (IS4) b = Unpack<QT, AT>::run(tl.q0[j], lut);
+                    if constexpr (IS4) b = Unpack<QT, AT>::run(tl.q0[j], lut, magic);
                     else if (j < 2) b = Unpack8<QT, AT>::run(tl.q0[2 * j], tl.q0[2 * j + 1]);
                     else b = Unpack8<QT, AT>::run(tl.q1[2 * (j - 2)], tl.q1[2 * (j - 2) + 1]);
                     float d, mn;
