@@ -113,7 +113,8 @@ int lowbit_dequantize(const void *w, void *dst, int qtype, int64_t N, int64_t K,
                       void *stream);
 /* xe_linear.forward_new / xe_batch.batch_forward (low_bit_linear.py:657-668, xpu_ops.py:23-26):
  * y[M, N] = x[M, K] * dequant(w)[N, K]^T, x and y of act_dtype (f16 or bf16), fp32 accumulation.
- * Picks the streaming GEMV for small M and the MFMA GEMM for large M. */
+ * Picks the streaming GEMV (one pass over the weights per 16 rows) or the MFMA GEMM, whichever it
+ * estimates to be faster for the shape. */
 int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
                    int64_t N, int64_t K, void *stream);
 /* The two kernels behind lowbit_forward, for callers (and benchmarks) that choose themselves.

@@ -148,10 +148,18 @@ int lowbit_gemm(const void *x, const void *w, void *y, int qtype, int layout, in
 
 int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
                    int64_t K, void *stream) {
-    // The GEMV streams the weights once for up to 16 rows of x; beyond that the MFMA GEMM
-    // (which needs the tiled layout) amortizes the dequantization over a 2-D tile.
+    // The GEMV streams the weights once per 16 rows of x; the MFMA GEMM (which needs the tiled
+    // layout) amortizes the dequantization over a 128 x 256 tile but walks K in steps that cost about
+    // 1.9 us each while the machine is not full - a lone row tile of [11008 x 4096] takes 61 us however
+    // few rows it holds, where a GEMV pass takes 12 us.  Both are estimated (constants measured on
+    // MI355X) and the cheaper one runs; the GEMV wins up to M of roughly 32 .. 128 depending on shape.
     if (M <= 16 || layout != LOWBIT_LAYOUT_TILED)
         return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
+    const double passes = (double)((M + 15) / 16);
+    const double t_gemv = passes * ((double)lowbit_blob_bytes(qtype, N * K) / 2.8e6 + 2.5);       // us
+    const double tiles = (double)((M + 127) / 128) * (double)((N + 255) / 256);
+    const double t_gemm = (double)(K / 128) * 1.9 * (tiles > 512.0 ? tiles / 512.0 : 1.0);        // us
+    if (t_gemv < t_gemm) return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
     return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);
 }
 
