@@ -350,11 +350,15 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream):
               for k in {k for _, k, _ in mods}}
         ys = {n: torch.empty((m, n), dtype=tdt, device=dev) for n, _, _ in mods}
 
+        # caller-owned workspace: lets the GEMM split K where the output tiles alone do not fill the GPU
+        ws_bytes = max(16, max(ggml.lowbit_workspace_bytes(m, n, k) for n, k, _ in mods))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
         def run():
             st = stream()
             for n, k, blob in mods:
-                ggml.lowbit_forward(xs[k].data_ptr(), blob.data_ptr(), ys[n].data_ptr(), qtype, ggml.LAYOUT_TILED,
-                                    dt, m, n, k, st)
+                ggml.lowbit_forward_ws(xs[k].data_ptr(), blob.data_ptr(), ys[n].data_ptr(), qtype, ggml.LAYOUT_TILED,
+                                       dt, m, n, k, ws.data_ptr(), ws_bytes, st)
         g = capture(run)
         ms = time_graph(g, reps, 2)
         flop = sum(2.0 * m * n * k for n, k, _ in mods)

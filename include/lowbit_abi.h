@@ -145,6 +145,19 @@ int lowbit_moe_forward(const void *x, const int32_t *topk_ids, const float *topk
                        const void *const *gates, const void *const *ups, const void *const *downs, void *workspace,
                        void *y, int qtype, int act_dtype, int64_t hidden, int64_t inter, int act, void *stream);
 
+/* The same products with a caller-owned workspace in device memory (16-byte aligned): the GEMM may
+ * then split K over more workgroups and sum fp32 partial tiles from the workspace in a second launch,
+ * which fills the machine when M is small or N narrow.  No counterpart in the reference (its closed
+ * kernels manage their own memory); lowbit_workspace_bytes says how much is worth passing for a
+ * shape (0: the workspace would not be used).  A smaller or null workspace is always valid. */
+size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int lowbit_forward_ws(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                      int64_t N, int64_t K, void *workspace, size_t workspace_bytes, void *stream);
+/* splits: 0 = the library's choice for the workspace given, n > 1 = exactly n K-splits (needs
+ * n * ceil(M/128) * ceil(N/256) * 128 KiB of workspace), 1 = none. */
+int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
+                   int64_t K, void *workspace, size_t workspace_bytes, int splits, void *stream);
+
 /* Grouped product for mixture-of-experts layers, one launch for all experts.  The reference has
  * no single call for it: it loops over the experts in Python and calls each expert's LowBitLinear
  * on the rows routed to it (python/llm/src/ipex_llm/transformers/models/qwen2_moe.py:375-430 is the

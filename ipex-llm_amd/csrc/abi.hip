@@ -21,7 +21,9 @@ int launch_dequantize(const void *w, void *out, int qtype, int64_t N, int64_t K,
 int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 int waves, hipStream_t st);
 int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
-                hipStream_t st);
+                void *workspace, size_t workspace_bytes, int want_splits, hipStream_t st);
+int gemm_splits(int M, int N, int K, size_t ws_bytes);
+double gemm_time_us(int M, int N, int K, int splits);
 int launch_grouped_gemm(const void *x, const void *const *w, void *y, const int32_t *offsets, int n_groups,
                         int total_rows, int qtype, int act_dtype, int N, int K, hipStream_t st);
 }  // namespace lowbit
@@ -137,30 +139,78 @@ int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, in
                                     (hipStream_t)stream), "lowbit_gemv");
 }
 
+static size_t split_bytes(int64_t M, int64_t N, int splits) {
+    return (size_t)splits * (size_t)((M + 127) / 128) * (size_t)((N + 255) / 256) * 128 * 256 * sizeof(float);
+}
+
+static int gemm_entry(const char *what, const void *x, const void *w, void *y, int qtype, int layout, int act_dtype,
+                      int64_t M, int64_t N, int64_t K, void *workspace, size_t workspace_bytes, int splits,
+                      void *stream) {
+    if (int rc = check_mm(what, x, w, y, qtype, layout, act_dtype, M, N, K)) return rc;
+    if (M * N == 0) return 0;
+    if (K == 0) return fail(LOWBIT_ESHAPE, "%s: K == 0", what);
+    if (workspace && !aligned16(workspace)) return fail(LOWBIT_EARG, "%s: workspace must be 16-byte aligned", what);
+    if (splits < 0 || splits > 64) return fail(LOWBIT_EARG, "%s: splits must be 0 (automatic) .. 64", what);
+    if (splits > 1) {
+        if (!workspace || split_bytes(M, N, splits) > workspace_bytes)
+            return fail(LOWBIT_ESIZE, "%s: %d splits need %zu bytes of workspace", what, splits, split_bytes(M, N, splits));
+        if (layout != LOWBIT_LAYOUT_TILED || splits > K / 128)
+            return fail(LOWBIT_ESHAPE, "%s: %d splits need the tiled layout and at least as many 128-column steps", what,
+                        splits);
+    }
+    return check_launch(launch_gemm(x, w, y, qtype, layout, act_dtype, (int)M, (int)N, (int)K, workspace,
+                                    workspace ? workspace_bytes : 0, splits, (hipStream_t)stream), what);
+}
+
 int lowbit_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
                 int64_t K, void *stream) {
-    if (int rc = check_mm("lowbit_gemm", x, w, y, qtype, layout, act_dtype, M, N, K)) return rc;
-    if (M * N == 0) return 0;
-    if (K == 0) return fail(LOWBIT_ESHAPE, "lowbit_gemm: K == 0");
-    return check_launch(launch_gemm(x, w, y, qtype, layout, act_dtype, (int)M, (int)N, (int)K, (hipStream_t)stream),
-                        "lowbit_gemm");
+    return gemm_entry("lowbit_gemm", x, w, y, qtype, layout, act_dtype, M, N, K, nullptr, 0, 0, stream);
+}
+
+int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
+                   int64_t K, void *workspace, size_t workspace_bytes, int splits, void *stream) {
+    return gemm_entry("lowbit_gemm_ws", x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, splits,
+                      stream);
+}
+
+size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;
+    const int s = gemm_splits((int)M, (int)N, (int)K, (size_t)-1);
+    return s > 1 ? split_bytes(M, N, s) : 0;
+}
+
+// Choice of kernel behind lowbit_forward, by estimated run time (constants measured on MI355X).  The
+// GEMV streams the weights once per 16 rows of x (about 2.8 TB/s plus 2.5 us per pass; later passes come
+// partly out of the Infinity Cache).  The MFMA GEMM amortizes the dequantization over 128 x 256 tiles
+// but is latency-bound while its tiles do not fill the machine: a lone row tile of [11008 x 4096] takes
+// 61 us however few rows it holds, where a GEMV pass takes 12 us.  With a workspace the GEMM can split
+// K over more workgroups at the price of writing and re-reading fp32 partial sums.
+static int forward_any(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                       int64_t N, int64_t K, void *workspace, size_t workspace_bytes, void *stream) {
+    if (M <= 16 || layout != LOWBIT_LAYOUT_TILED)
+        return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
+    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || K < 128)
+        return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);     // reports the error
+    const double passes = (double)((M + 15) / 16);
+    const double t_gemv = passes * ((double)lowbit_blob_bytes(qtype, N * K) / 2.8e6 + 2.5);
+    const int splits = workspace ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
+    const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits);
+    if (t_gemv < t_gemm) return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
+    if (splits > 1)
+        return lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, splits, stream);
+    return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);
 }
 
 int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
                    int64_t K, void *stream) {
-    // The GEMV streams the weights once per 16 rows of x; the MFMA GEMM (which needs the tiled
-    // layout) amortizes the dequantization over a 128 x 256 tile but walks K in steps that cost about
-    // 1.9 us each while the machine is not full - a lone row tile of [11008 x 4096] takes 61 us however
-    // few rows it holds, where a GEMV pass takes 12 us.  Both are estimated (constants measured on
-    // MI355X) and the cheaper one runs; the GEMV wins up to M of roughly 32 .. 128 depending on shape.
-    if (M <= 16 || layout != LOWBIT_LAYOUT_TILED)
-        return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
-    const double passes = (double)((M + 15) / 16);
-    const double t_gemv = passes * ((double)lowbit_blob_bytes(qtype, N * K) / 2.8e6 + 2.5);       // us
-    const double tiles = (double)((M + 127) / 128) * (double)((N + 255) / 256);
-    const double t_gemm = (double)(K / 128) * 1.9 * (tiles > 512.0 ? tiles / 512.0 : 1.0);        // us
-    if (t_gemv < t_gemm) return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
-    return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);
+    return forward_any(x, w, y, qtype, layout, act_dtype, M, N, K, nullptr, 0, stream);
+}
+
+int lowbit_forward_ws(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
+                      int64_t K, void *workspace, size_t workspace_bytes, void *stream) {
+    if (workspace && !aligned16(workspace))
+        return fail(LOWBIT_EARG, "lowbit_forward_ws: workspace must be 16-byte aligned");
+    return forward_any(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace ? workspace_bytes : 0, stream);
 }
 
 int lowbit_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, void *dst, int qtype, int64_t N,

@@ -193,7 +193,8 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
                                                         AT *__restrict__ y, int M, int N, int K, int xcd_m,
                                                         const int32_t *__restrict__ group_offsets,
                                                         const uint8_t *const *__restrict__ group_weights,
-                                                        int n_groups, int max_mtiles) {
+                                                        int n_groups, int max_mtiles, int k_steps,
+                                                        float *__restrict__ ws) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
     // x block in operand order: [16-column step ks (8)][32-row block (MB32)][lane (64)] x 16 bytes
@@ -284,9 +285,14 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             xoff[mb] = (uint32_t)(((int64_t)row * K + kg * 8) * (int64_t)sizeof(AT));
         }
     }
-    const int last = G - 1;
+    // Split-K: with a workspace the grid has a second dimension, workgroup (t, s) walks the K steps
+    // s * k_steps .. and leaves its fp32 partial tile in ws[s]; a second kernel sums the splits.  It
+    // fills the machine when the output alone has too few tiles (small M, narrow N).
+    const int kt0 = ws ? blockIdx.y * k_steps : 0;
+    const int Gs = ws ? (k_steps < G - kt0 ? k_steps : G - kt0) : G;
+    const int last = Gs - 1;
     auto dma_x = [&](int kt, uint8_t *buf) {
-        kt = kt < last ? kt : last;
+        kt = kt0 + (kt < last ? kt : last);
         const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT) + wave * 2 * 16 * sizeof(AT);
         // Issued from inline assembly: the compiler's wait-count pass treats an LDS-DMA as aliasing
         // every later LDS access and would wait for it immediately.  Completion is awaited by the
@@ -301,7 +307,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         }
     };
     auto load_x = [&](int kt, u32x4 (&xr)[8]) {
-        kt = kt < last ? kt : last;                      // past the end: a harmless re-read, never used
+        kt = kt0 + (kt < last ? kt : last);              // past the end: a harmless re-read, never used
         const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
 #pragma unroll
         for (int i = 0; i < 8; i++) xr[i] = *(const u32x4 *)(xk + xoff[i]);
@@ -314,7 +320,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         TileRegs<QT> lo[NB32], hi[NB32];
     };
     auto load_w = [&](int kt, WRegs &t) {
-        kt = kt < last ? kt : last;
+        kt = kt0 + (kt < last ? kt : last);
 #pragma unroll
         for (int nb = 0; nb < NB32; nb++) {
             const gbytes tile = wt[nb] + (int64_t)kt * F::TILE_BYTES;
@@ -410,11 +416,23 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
                 for (int q = 0; q < 4; q++) {
                     const int n = n0 + nb * 32 + q * 8 + kg * 4;
                     if (n < N) {
-                        typedef AT at4 __attribute__((ext_vector_type(4)));
-                        at4 o;
+                        if (ws) {
+                            // partial sums keep the register layout (split, tile, wave, register group,
+                            // lane): every store is 1 KiB contiguous; the reduction kernel undoes it
+                            const f32x4 o = {acc[mb][nb][q * 4], acc[mb][nb][q * 4 + 1], acc[mb][nb][q * 4 + 2],
+                                             acc[mb][nb][q * 4 + 3]};
+                            const int64_t tile_id = (int64_t)(m0 / GM) * ((N + GN - 1) / GN) + tile_n;
+                            const int64_t n_tiles_all = (int64_t)((M + GM - 1) / GM) * ((N + GN - 1) / GN);
+                            const int64_t slot = (((int64_t)blockIdx.y * n_tiles_all + tile_id) * 4 + wave) * (MB32 * NB32 * 4) +
+                                                 (mb * NB32 + nb) * 4 + q;
+                            *(f32x4 *)(ws + (slot * 64 + lane) * 4) = o;
+                        } else {
+                            typedef AT at4 __attribute__((ext_vector_type(4)));
+                            at4 o;
 #pragma unroll
-                        for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
-                        *(at4 *)(y + (int64_t)m * N + n) = o;
+                            for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
+                            *(at4 *)(y + (int64_t)m * N + n) = o;
+                        }
                     }
                 }
                 // one 32x32 block at a time: moving all 128 accumulators to vector registers at
@@ -436,7 +454,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             load_w(0, w0);
             wait_all_loads();
             __syncthreads();
-            for (int kt = 0; kt + 1 < G; kt += 2) {
+            for (int kt = 0; kt + 1 < Gs; kt += 2) {
                 dma_x(kt + 1, xs1);
                 load_w(kt + 1, w1);
                 compute(xs0, w0, mbc);
@@ -448,7 +466,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
                 wait_all_loads();
                 __syncthreads();
             }
-            if (G & 1) compute(xs0, w0, mbc);
+            if (Gs & 1) compute(xs0, w0, mbc);
         };
         // tail tiles and small expert groups: 32-row blocks without rows of x skip their MFMAs
         const int mb_cnt = (M - m0 + 31) / 32;
@@ -477,14 +495,14 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
     __syncthreads();
 
 #define LOWBIT_GEMM_STEP(i, cur, nxt, xst, xld, wc, wl) \
-    if (kt + (i) < G) {                                 \
+    if (kt + (i) < Gs) {                                \
         load_x(kt + (i) + 2, xld);                      \
         load_w(kt + (i) + 2, wl);                       \
         compute(cur, wc, full_t());                     \
         store_x(nxt, xst);                              \
         __syncthreads();                                \
     }
-    for (int kt = 0; kt < G; kt += 6) {
+    for (int kt = 0; kt < Gs; kt += 6) {
         LOWBIT_GEMM_STEP(0, xs0, xs1, xb, xa, w0, w2)
         LOWBIT_GEMM_STEP(1, xs1, xs0, xa, xb, w1, w0)
         LOWBIT_GEMM_STEP(2, xs0, xs1, xb, xa, w2, w1)
@@ -498,25 +516,105 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
 }
 
 
+// Sums the fp32 partial tiles of the splits (stored in the GEMM's register layout: split, tile, wave,
+// register group, lane) and writes y, rounded once.  One thread per group of 4 consecutive n.
+template <typename AT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ ws, AT *__restrict__ y, int M,
+                                                            int N, int splits) {
+    const int tiles_n = (N + GN - 1) / GN;
+    const int64_t n_tiles_all = (int64_t)((M + GM - 1) / GM) * tiles_n;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;       // (tile, wave, group, lane)
+    if (t >= n_tiles_all * 4 * (MB32 * NB32 * 4) * 64) return;
+    const int lane = (int)(t & 63);
+    const int grp = (int)((t >> 6) % (MB32 * NB32 * 4));
+    const int wave = (int)((t >> 6) / (MB32 * NB32 * 4) % 4);
+    const int64_t tile_id = (t >> 6) / (MB32 * NB32 * 4) / 4;
+    const int mb = grp / (NB32 * 4), nb = grp / 4 % NB32, q = grp % 4;
+    const int m = (int)(tile_id / tiles_n) * GM + mb * 32 + (lane & 31);
+    const int n = (int)(tile_id % tiles_n) * GN + wave * GN_WAVE + nb * 32 + q * 8 + (lane >> 5) * 4;
+    if (m >= M || n >= N) return;
+    const int64_t per_split = n_tiles_all * 4 * (MB32 * NB32 * 4) * 64 * 4;     // floats
+    f32x4 a = *(const f32x4 *)(ws + t * 4);
+    for (int s = 1; s < splits; s++) a += *(const f32x4 *)(ws + (int64_t)s * per_split + t * 4);
+    typedef AT at4 __attribute__((ext_vector_type(4)));
+    at4 o;
+#pragma unroll
+    for (int k = 0; k < 4; k++) o[k] = to_at<AT>(a[k]);
+    *(at4 *)(y + (int64_t)m * N + n) = o;
+}
+
+// Estimated run time in microseconds of the GEMM with K split `splits` ways (1 = no split), from
+// measurements on MI355X: a workgroup takes about 1.9 us per 128-column step on an otherwise idle
+// machine, 2.7 us when every CU holds one workgroup and 5.0 us when every CU holds two (the clock
+// drops and the memory system fills as more CUs work); the partial sums of a split are written and
+// read back at about 4 TB/s.
+double gemm_time_us(int M, int N, int K, int splits) {
+    const double tiles = (double)((M + GM - 1) / GM) * (double)((N + GN - 1) / GN);
+    const int G = K / TILE_COLS;
+    const int k_steps = (G + splits - 1) / splits;
+    const int ny = (G + k_steps - 1) / k_steps;
+    const double wgs = tiles * ny;
+    const double live = wgs < 512.0 ? wgs : 512.0;
+    // row tiles that are partly empty skip MFMAs and write fewer partial sums: the load-dependent
+    // part of a step and the reduction traffic shrink with the fill, the latency floor does not
+    const double fill = (double)M / ((double)((M + GM - 1) / GM) * GM);
+    const double load = live <= 256.0 ? 0.8 * live / 256.0 : 0.8 + 2.3 * (live - 256.0) / 256.0;
+    const double step = 1.9 + load * (0.4 + 0.6 * fill);
+    double t = (double)k_steps * step * (wgs > 512.0 ? wgs / 512.0 : 1.0);
+    if (ny > 1) t += (double)ny * tiles * (GM * GN * 8.0) * fill / 4.0e6 + 3.0;
+    return t;
+}
+
+// Number of K splits to use for this shape given `ws_bytes` of workspace (1 = none): the fastest by
+// the estimate above among 1 .. 8 splits of at least two K steps that fit the workspace.
+int gemm_splits(int M, int N, int K, size_t ws_bytes) {
+    const size_t tiles = (size_t)((M + GM - 1) / GM) * (size_t)((N + GN - 1) / GN);
+    const size_t per_split = tiles * GM * GN * sizeof(float);     // whole tiles: partial sums keep the tile layout
+    const int G = K / TILE_COLS;
+    int best = 1;
+    double best_t = gemm_time_us(M, N, K, 1);
+    for (int s = 2; s <= 8 && s * 2 <= G; s++) {
+        if ((size_t)s * per_split > ws_bytes) break;
+        const double t = gemm_time_us(M, N, K, s);
+        if (t < 0.9 * best_t) {                                   // a split must pay clearly
+            best = s;
+            best_t = t;
+        }
+    }
+    return best;
+}
+
 template <int QT, typename AT>
-static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, int K, hipStream_t st) {
+static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, int K, float *ws, int splits,
+                         hipStream_t st) {
     const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
     int xcd_m = 1;                                       // XCDs along M: power of two <= min(8, tiles_m)
     while (xcd_m * 2 <= 8 && xcd_m * 2 <= tiles_m) xcd_m *= 2;
     const int xcd_n = 8 / xcd_m;
     const int band_m = (tiles_m + xcd_m - 1) / xcd_m, band_n = (tiles_n + xcd_n - 1) / xcd_n;
-    dim3 grid(8 * band_m * band_n);
+    if (splits <= 1) ws = nullptr;
+    const int G = K / TILE_COLS;
+    const int k_steps = ws ? (G + splits - 1) / splits : G;
+    const int ny = ws ? (G + k_steps - 1) / k_steps : 1;             // splits that actually hold steps
+    dim3 grid(8 * band_m * band_n, ny);
     // Two forms of the kernel.  The DMA form (x straight into LDS, one K step of prefetch, 128
     // vector registers) lets a CU hold two workgroups that cover each other's waits; it wins as
-    // soon as there are more tiles than CUs.  With at most one tile per CU the register-staged
+    // soon as there are more workgroups than CUs.  With at most one per CU the register-staged
     // form with its deeper prefetch is faster.
-    const bool dma = tiles_m * tiles_n > 256;
+    const bool dma = tiles_m * tiles_n * ny > 256;
     if (dma)
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
-                           (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0);
+                           (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0,
+                           k_steps, ws);
     else
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, false>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
-                           (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0);
+                           (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0,
+                           k_steps, ws);
+    if (ws) {
+        const int64_t threads = (int64_t)tiles_m * tiles_n * (GM * GN / 4);
+        hipLaunchKernelGGL((splitk_reduce_kernel<AT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, ws,
+                           (AT *)y, M, N, ny);
+    }
     return 0;
 }
 
@@ -527,7 +625,7 @@ static int launch_grouped_t(const void *x, const void *const *w, void *y, const 
     const int tiles_n = (N + GN - 1) / GN;
     hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true>), dim3(tiles_n * max_mtiles), dim3(256), 0, st, (const AT *)x,
                        (const uint8_t *)nullptr, (AT *)y, 0, N, K, 1, offsets, (const uint8_t *const *)w, n_groups,
-                       max_mtiles);
+                       max_mtiles, 0, (float *)nullptr);
     return 0;
 }
 
@@ -554,25 +652,29 @@ int launch_grouped_gemm(const void *x, const void *const *w, void *y, const int3
 }
 
 template <int QT>
-static int launch_gemm_q(const void *x, const void *w, void *y, int dt, int M, int N, int K, hipStream_t st) {
-    if (dt == DT_F16) return launch_gemm_t<QT, _Float16>(x, w, y, M, N, K, st);
-    if (dt == DT_BF16) return launch_gemm_t<QT, __bf16>(x, w, y, M, N, K, st);
+static int launch_gemm_q(const void *x, const void *w, void *y, int dt, int M, int N, int K, float *ws, int splits,
+                         hipStream_t st) {
+    if (dt == DT_F16) return launch_gemm_t<QT, _Float16>(x, w, y, M, N, K, ws, splits, st);
+    if (dt == DT_BF16) return launch_gemm_t<QT, __bf16>(x, w, y, M, N, K, ws, splits, st);
     return -4;
 }
 
+// splits: 0 = chosen here from the workspace size, otherwise as given (the caller has checked that it fits)
 int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
-                hipStream_t st) {
+                void *workspace, size_t workspace_bytes, int want_splits, hipStream_t st) {
     if (M == 0 || N == 0) return 0;
     // the MFMA GEMM reads the tiled layout and stores 8-byte groups of y (N % 4 == 0 is implied
     // by N % 16 == 0); anything else goes through the streaming kernel in 16-row slices
     if (layout != LAYOUT_TILED || (N % TILE_ROWS) || (K % TILE_COLS) || (((uintptr_t)y) & 7))
         return launch_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, st);
+    float *ws = (float *)workspace;
+    const int splits = !ws ? 1 : want_splits > 0 ? want_splits : gemm_splits(M, N, K, workspace_bytes);
     switch (qtype) {
-    case QT_SYM_INT4: return launch_gemm_q<QT_SYM_INT4>(x, w, y, act_dtype, M, N, K, st);
-    case QT_ASYM_INT4: return launch_gemm_q<QT_ASYM_INT4>(x, w, y, act_dtype, M, N, K, st);
-    case QT_SYM_INT8: return launch_gemm_q<QT_SYM_INT8>(x, w, y, act_dtype, M, N, K, st);
-    case QT_NF4: return launch_gemm_q<QT_NF4>(x, w, y, act_dtype, M, N, K, st);
-    case QT_FP8_E4M3: return launch_gemm_q<QT_FP8_E4M3>(x, w, y, act_dtype, M, N, K, st);
+    case QT_SYM_INT4: return launch_gemm_q<QT_SYM_INT4>(x, w, y, act_dtype, M, N, K, ws, splits, st);
+    case QT_ASYM_INT4: return launch_gemm_q<QT_ASYM_INT4>(x, w, y, act_dtype, M, N, K, ws, splits, st);
+    case QT_SYM_INT8: return launch_gemm_q<QT_SYM_INT8>(x, w, y, act_dtype, M, N, K, ws, splits, st);
+    case QT_NF4: return launch_gemm_q<QT_NF4>(x, w, y, act_dtype, M, N, K, ws, splits, st);
+    case QT_FP8_E4M3: return launch_gemm_q<QT_FP8_E4M3>(x, w, y, act_dtype, M, N, K, ws, splits, st);
     default: return -2;
     }
 }

@@ -176,6 +176,30 @@ _lib.lowbit_gemm.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, 
 _lib.lowbit_gemm.restype = c_int
 
 
+_lib.lowbit_workspace_bytes.argtypes = [c_int64, c_int64, c_int64]
+_lib.lowbit_workspace_bytes.restype = c_size_t
+_lib.lowbit_forward_ws.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
+                                   c_void_p, c_size_t, c_void_p]
+_lib.lowbit_forward_ws.restype = c_int
+_lib.lowbit_gemm_ws.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
+                                c_void_p, c_size_t, c_int, c_void_p]
+_lib.lowbit_gemm_ws.restype = c_int
+
+
+def lowbit_workspace_bytes(m, n, k) -> int:
+    return _lib.lowbit_workspace_bytes(m, n, k)
+
+
+def lowbit_forward_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, stream):
+    _check(_lib.lowbit_forward_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, stream),
+           "lowbit_forward_ws")
+
+
+def lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, splits, stream):
+    _check(_lib.lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, splits, stream),
+           "lowbit_gemm_ws")
+
+
 _lib.lowbit_grouped_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int,
                                         c_int64, c_int64, c_void_p]
 _lib.lowbit_grouped_forward.restype = c_int

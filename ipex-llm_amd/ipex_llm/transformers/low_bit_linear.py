@@ -40,6 +40,7 @@ FP16 = ggml_tensor_qtype["fp16"]
 BF16 = ggml_tensor_qtype["bf16"]
 
 _ACCEL = "cuda"   # device.type of an MI355X under PyTorch-ROCm
+_WORKSPACE_CAP = 256 << 20   # most that forward_new borrows for split-K partial sums
 _DT = {torch.float16: ggml.DT_F16, torch.bfloat16: ggml.DT_BF16, torch.float32: ggml.DT_F32}
 
 
@@ -231,8 +232,17 @@ def forward_new(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int, 
     y = torch.empty((m, output_size), dtype=xc.dtype, device=x.device)
     if m and output_size:
         with torch.cuda.device(x.device):
-            ggml.lowbit_forward(xc.data_ptr(), w.data_ptr(), y.data_ptr(), qtype, layout, _DT[xc.dtype],
-                                m, output_size, k, _stream())
+            # split-K workspace for shapes whose output tiles alone do not fill the GPU; taken from
+            # torch's caching allocator, so steady-state calls do not allocate
+            ws_bytes = ggml.lowbit_workspace_bytes(m, output_size, k) if layout == ggml.LAYOUT_TILED else 0
+            ws_bytes = min(ws_bytes, _WORKSPACE_CAP)
+            if ws_bytes:
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+                ggml.lowbit_forward_ws(xc.data_ptr(), w.data_ptr(), y.data_ptr(), qtype, layout, _DT[xc.dtype],
+                                       m, output_size, k, ws.data_ptr(), ws_bytes, _stream())
+            else:
+                ggml.lowbit_forward(xc.data_ptr(), w.data_ptr(), y.data_ptr(), qtype, layout, _DT[xc.dtype],
+                                    m, output_size, k, _stream())
     return y if y.dtype == x.dtype else y.to(x.dtype)
 
 

@@ -288,3 +288,41 @@ def test_llama3_70b_shapes_decode_against_oracle(qtype, n, k, m):
     y = dev_matmul(x, blob, qtype, TILED, n)
     y_exact = orc.mul_mat_exact(orc.quantize(w, qtype), x.float().numpy(), (n, k), qtype)
     assert np.abs(y - y_exact).max() <= 8e-3 * np.abs(y_exact).max()
+
+
+@pytest.mark.parametrize("qtype,dtype", [(Q4_0, torch.float16), (Q8_0, torch.bfloat16), (NF4, torch.bfloat16)])
+@pytest.mark.parametrize("m,n,k,splits", [(48, 1024, 4096, 8), (200, 272, 1408, 3), (512, 4096, 2048, 2),
+                                          (130, 11008, 1024, 4), (300, 7168, 896, 7)])
+def test_split_k_gemm_against_oracle(qtype, dtype, m, n, k, splits):
+    # K split over several workgroups per tile, partial sums through a workspace; ragged splits
+    # (11 steps in 3, 7 steps in 7), both forms of the kernel, tail row tiles
+    w = weights(5500 + qtype + m, (n, k))
+    x = acts(5501 + m, m, k, dtype)
+    blob = dev_quantize(w, qtype, TILED)
+    xd = x.cuda()
+    ws_bytes = splits * -(-m // 128) * -(-n // 256) * 128 * 256 * 4
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+
+    def run(entry, *tail):
+        y = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        entry(xd.data_ptr(), blob.data_ptr(), y.data_ptr(), qtype, TILED, DT[dtype], m, n, k, *tail, stream())
+        torch.cuda.synchronize()
+        return y.float().cpu().numpy()
+    y = run(ggml.lowbit_gemm_ws, ws.data_ptr(), ws_bytes, splits)
+    y_exact = orc.mul_mat_exact(orc.quantize(w, qtype), x.float().numpy(), (n, k), qtype)
+    tol = 2e-3 if dtype == torch.float16 else 8e-3
+    assert np.isfinite(y).all() and np.abs(y - y_exact).max() <= tol * np.abs(y_exact).max()
+    # one split is the plain kernel, bit for bit; an automatic choice and forward agree with the oracle too
+    assert np.array_equal(run(ggml.lowbit_gemm_ws, ws.data_ptr(), ws_bytes, 1), dev_matmul(x, blob, qtype, TILED, n, fn="gemm"))
+    for y_auto in (run(ggml.lowbit_gemm_ws, ws.data_ptr(), ws_bytes, 0), run(ggml.lowbit_forward_ws, ws.data_ptr(), ws_bytes)):
+        assert np.abs(y_auto - y_exact).max() <= tol * np.abs(y_exact).max()
+    with pytest.raises(RuntimeError, match="workspace"):
+        run(ggml.lowbit_gemm_ws, ws.data_ptr(), ws_bytes - 16, splits)
+
+
+def test_workspace_query_is_consistent():
+    for m, n, k in [(256, 4096, 11008), (64, 28672, 8192), (2048, 11008, 4096), (8, 4096, 4096)]:
+        b = ggml.lowbit_workspace_bytes(m, n, k)
+        assert b % (128 * 256 * 4) == 0
+    assert ggml.lowbit_workspace_bytes(256, 4096, 11008) > 0        # 32 tiles, 86 steps: worth splitting
+    assert ggml.lowbit_workspace_bytes(2048, 11008, 4096) == 0      # 688 tiles fill the machine
