@@ -226,7 +226,7 @@ def main():
                 "frac": round(hb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counters of this very loop
                 # (profiles/gemv_sym_int4_f16_N11008_K4096_M1.md); valid for M = 1 only
-                "traffic": 25510035 if args.m == 1 else None,
+                "traffic": 25496723 if args.m == 1 else None,
                 "bytes_per_launch": hb, "avg_launch_us": round(us, 3),
                 "how": "HIP events around graph replays of 64 chained launches over 64 distinct weights"}
     if args.roofline_only:
