@@ -211,3 +211,34 @@ def test_training_backward_is_grad_out_times_the_dequantized_weight(qname, dtype
     assert x.grad.shape == x.shape and x.grad.dtype == dtype
     assert (x.grad.float() - want).abs().max() <= 1e-2 * want.abs().max()
     assert layer.weight.grad is None
+
+
+def test_lowbit_linears_replay_correctly_from_a_hip_graph():
+    """Decode and small-prefill calls captured once and replayed with new inputs (static buffers), with
+    eager work and synchronizations between the replays; every replay must equal the eager result."""
+    torch.manual_seed(9)
+    lins = [_layer(weights(7200 + i, (n, k)), Q["sym_int4"]).to("cuda") for i, (n, k) in
+            enumerate([(512, 256), (256, 512)])]
+    emb_like = _layer(weights(7210, (4096, 256)), Q["sym_int8"]).to("cuda")      # many tiles, long K walk
+
+    def net(x):
+        return emb_like(lins[1](torch.nn.functional.silu(lins[0](x))))
+    for rows in (1, 48):                                   # GEMV path / split-K GEMM path with a workspace
+        static_x = torch.zeros(rows, 256, dtype=torch.float16, device="cuda")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            net(static_x)                                  # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = net(static_x)
+        for step in range(4):
+            x = torch.randn(rows, 256, device="cuda").half()
+            want = net(x)                                  # eager work between the replays
+            torch.cuda.synchronize()
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want), (rows, step)
