@@ -174,7 +174,7 @@ int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout,
 }
 
 size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;
+    if (M <= 16 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;   // M <= 16: GEMV
     const int s = gemm_splits((int)M, (int)N, (int)K, (size_t)-1);
     return s > 1 ? split_bytes(M, N, s) : 0;
 }
