@@ -108,7 +108,8 @@ int lowbit_quantize(const float *src, void *dst, int qtype, int64_t N, int64_t K
 /* ggml_q_format_convet_cpu2xpu / _xpu2cpu with the shape: src in `src_layout` -> dst in the
  * other layout.  src and dst must not overlap. */
 int lowbit_relayout(const void *src, void *dst, int qtype, int64_t N, int64_t K, int src_layout, void *stream);
-/* xe_linear.dequant (low_bit_linear.py:534-538) / ggml_dequantize: blob -> dense [N, K]. */
+/* xe_linear.dequant (low_bit_linear.py:534-538) / ggml_dequantize: blob -> dense [N, K].  dst is
+ * 16-byte aligned (so is dst of lowbit_dequantize_rows). */
 int lowbit_dequantize(const void *w, void *dst, int qtype, int64_t N, int64_t K, int layout, int out_dtype,
                       void *stream);
 /* xe_linear.forward_new / xe_batch.batch_forward (low_bit_linear.py:657-668, xpu_ops.py:23-26):

@@ -112,7 +112,8 @@ int lowbit_dequantize(const void *w, void *dst, int qtype, int64_t N, int64_t K,
                       void *stream) {
     if (int rc = check_weight_shape("lowbit_dequantize", qtype, N, K, layout)) return rc;
     if (N * K == 0) return 0;
-    if (!w || !dst || !aligned16(w)) return fail(LOWBIT_EARG, "lowbit_dequantize: null or misaligned pointer");
+    if (!w || !dst || !aligned16(w) || !aligned16(dst))
+        return fail(LOWBIT_EARG, "lowbit_dequantize: null or misaligned pointer");
     return check_launch(launch_dequantize(w, dst, qtype, N, K, layout, out_dtype, (hipStream_t)stream),
                         "lowbit_dequantize");
 }
@@ -218,7 +219,7 @@ int lowbit_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, v
     if (int rc = check_weight_shape("lowbit_dequantize_rows", qtype, N, K, layout)) return rc;
     if (n_rows < 0) return fail(LOWBIT_EARG, "lowbit_dequantize_rows: negative row count");
     if (n_rows * K == 0) return 0;
-    if (!w || !rows || !dst || !aligned16(w))
+    if (!w || !rows || !dst || !aligned16(w) || !aligned16(dst))
         return fail(LOWBIT_EARG, "lowbit_dequantize_rows: null or misaligned pointer");
     return check_launch(launch_dequantize_rows(w, rows, n_rows, dst, qtype, N, K, layout, out_dtype,
                                                (hipStream_t)stream), "lowbit_dequantize_rows");

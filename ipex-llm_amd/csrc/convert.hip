@@ -84,31 +84,61 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict_
     // rows == nullptr: output row i is weight row i.  Otherwise output row i is weight row rows[i]
     // (xe_linear.dequantize_rows, python/llm/src/ipex_llm/transformers/embedding.py:218-221); an
     // index outside [0, N) gives a row of zeros.
+    // Every lane produces 16 bytes of output (4 fp32 or 8 16-bit columns) and loads only the bytes
+    // that hold its own codes; adjacent lanes cover adjacent columns, so a wave stores 1 KiB runs.
+    constexpr int CPL = 16 / (int)sizeof(OT), LPS = 32 / CPL;  // columns per lane, lanes per sub-block
+    __shared__ float cb[16];
+    if constexpr (QT == QT_NF4) {
+        // divergent lookups: LDS serves them at full rate, the constant cache does not
+        if (threadIdx.x < 16) cb[threadIdx.x] = NF4_CODEBOOK[threadIdx.x];
+        __syncthreads();
+    }
     const int64_t sbpr = K / 32;
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n_out * sbpr) return;
-    const int64_t i_out = t / sbpr;
-    const int64_t n = rows ? rows[i_out] : i_out;
-    const int sb = (int)(t % sbpr);
-    if (n < 0 || n >= N) {
-        OT *o = out + i_out * K + (int64_t)sb * 32;
-#pragma unroll
-        for (int i = 0; i < 32; i++) o[i] = from_f32<OT>(0.0f);
-        return;
+    if (t >= n_out * sbpr * LPS) return;
+    int lp = (int)(t % LPS);
+    int64_t i_out = (t / LPS) / sbpr;
+    int sb = (int)((t / LPS) % sbpr);
+    if constexpr (LAYOUT == LAYOUT_TILED && sizeof(OT) == 2) {
+        if (!rows) {
+            // whole matrix, 16-bit output: a workgroup covers one 16 x 128 tile, so that each line of
+            // the tile is fetched by one compute unit only (fp32 output measured no gain from it)
+            const int64_t wg_per_band = K / (16 * CPL);
+            const int64_t col = (blockIdx.x % wg_per_band) * (16 * CPL) + (threadIdx.x % 16) * CPL;
+            i_out = (blockIdx.x / wg_per_band) * TILE_ROWS + threadIdx.x / 16;
+            sb = (int)(col / 32);
+            lp = (int)(col % 32) / CPL;
+        }
     }
-    SubBlock s;
-    if constexpr (LAYOUT == LAYOUT_GGML) ggml_load_sub<QT>(w, n, K, sb, s);
-    else tiled_load_sub<QT>(w, n, K, sb, s);
-    OT *o = out + i_out * K + (int64_t)sb * 32;
+    const int64_t n = rows ? rows[i_out] : i_out;
+    typedef OT otv __attribute__((ext_vector_type(CPL)));
+    otv v;
 #pragma unroll
-    for (int i = 0; i < 32; i++) o[i] = from_f32<OT>(decode<QT>(s.code[i], s.d, s.m));
+    for (int i = 0; i < CPL; i++) v[i] = from_f32<OT>(0.0f);
+    if (n >= 0 && n < N) {
+#pragma unroll
+        for (int q = 0; q < CPL / 4; q++) {
+            uint32_t code[4], hdr;
+            const int part = lp * (CPL / 4) + q;
+            if constexpr (LAYOUT == LAYOUT_GGML) ggml_load4<QT>(w, n, K, sb, part, code, hdr);
+            else tiled_load4<QT>(w, n, K, sb, part, code, hdr);
+            float d, m;
+            hdr_to_scale<QT>(hdr, d, m);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if constexpr (QT == QT_NF4) v[q * 4 + i] = from_f32<OT>(cb[code[i]] * d);
+                else v[q * 4 + i] = from_f32<OT>(decode<QT>(code[i], d, m));
+            }
+        }
+    }
+    *(otv *)(out + i_out * K + (int64_t)sb * 32 + lp * CPL) = v;
 }
 
 template <int QT, typename OT>
 static int launch_dq2(const void *w, void *out, int64_t N, int64_t K, int layout, hipStream_t st, const int64_t *rows,
                       int64_t n_rows) {
     const int64_t n_out = rows ? n_rows : N;
-    const int64_t threads = n_out * (K / 32);
+    const int64_t threads = n_out * (K / 32) * (2 * (int64_t)sizeof(OT));  // one lane per 16 output bytes
     if (threads == 0) return 0;
     const int64_t grid = (threads + 255) / 256;
     if (grid > 0x7fffffff) return -3;

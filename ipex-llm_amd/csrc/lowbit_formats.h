@@ -253,6 +253,56 @@ __device__ inline void tiled_store_hdr(uint8_t *w, int64_t n, int64_t K, int sb,
     else *(uint32_t *)h = hdr;
 }
 
+// Four consecutive columns (4*part .. 4*part+3, part = 0..7) of sub-block sb of row n, and the raw
+// header of their block: what one lane of the dequantizers needs.
+template <int QT>
+__device__ inline void ggml_load4(const uint8_t *w, int64_t n, int64_t K, int sb, int part, uint32_t (&code)[4],
+                                  uint32_t &hdr) {
+    using F = Fmt<QT>;
+    constexpr int SPB = F::QK / 32;
+    const int64_t blk = n * (K / F::QK) + sb / SPB;
+    const uint8_t *b = w + blk * F::TS;
+    if constexpr (F::HDR == 2) hdr = (uint32_t)b[0] | ((uint32_t)b[1] << 8);
+    else hdr = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
+    // blocks are 18, 20, 34 or 132 bytes long and the codes start 2 or 4 bytes in: every 4-byte
+    // group of codes is 2-byte aligned
+    const uint8_t *q = b + F::HDR;
+    int off, sh = 0;
+    if constexpr (QT == QT_SYM_INT4 || QT == QT_ASYM_INT4) {
+        off = (part & 3) * 4; sh = (part >> 2) * 4;           // columns 16..31 sit in the high nibbles
+    } else if constexpr (QT == QT_NF4) {
+        off = part * 4; sh = (sb % SPB) * 4;                  // elements 32..63 sit in the high nibbles
+    } else {
+        off = (sb % SPB) * 32 + part * 4;
+    }
+    const uint16_t *q2 = (const uint16_t *)(q + off);
+    const uint32_t v = ((uint32_t)q2[0] | ((uint32_t)q2[1] << 16)) >> sh;
+    constexpr uint32_t MASK = F::BITS == 4 ? 0xfu : 0xffu;
+#pragma unroll
+    for (int i = 0; i < 4; i++) code[i] = (v >> (8 * i)) & MASK;
+}
+
+template <int QT>
+__device__ inline void tiled_load4(const uint8_t *w, int64_t n, int64_t K, int sb, int part, uint32_t (&code)[4],
+                                   uint32_t &hdr) {
+    using F = Fmt<QT>;
+    const uint8_t *t = w + tile_offset<QT>(n, K, sb);
+    const int r = (int)(n % TILE_ROWS), j = sb % 4;
+    const uint8_t *h = t + tile_hdr_offset<QT>(r, j);
+    if constexpr (F::HDR == 2) hdr = *(const uint16_t *)h;
+    else hdr = *(const uint32_t *)h;
+    const int lane = (part >> 1) * 16 + r, half = part & 1;
+    if constexpr (F::BITS == 4) {
+        // nibble order 0,2,4,6,1,3,5,7: columns 4*half .. +3 are nibbles 2*half, 2*half+4, 2*half+1, 2*half+5
+        const uint32_t v = *(const uint32_t *)(t + lane * 16 + j * 4) >> (8 * half);
+        code[0] = v & 0xf; code[1] = (v >> 16) & 0xf; code[2] = (v >> 4) & 0xf; code[3] = (v >> 20) & 0xf;
+    } else {
+        const uint32_t v = *(const uint32_t *)(t + (j / 2) * 1024 + lane * 16 + (j % 2) * 8 + half * 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) code[i] = (v >> (8 * i)) & 0xff;
+    }
+}
+
 // Stores one sub-block into the ggml layout (codes only for the part it covers;
 // the header when it is the first sub-block of its block).
 template <int QT>
