@@ -159,6 +159,9 @@ int lowbit_forward_ws(const void *x, const void *w, void *y, int qtype, int layo
 int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
                    int64_t K, void *workspace, size_t workspace_bytes, int splits, void *stream);
 
+int lowbit_gemm_ring(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
+                     int64_t K, void *workspace, size_t workspace_bytes, int wgs, int waves, void *stream);
+
 /* Grouped product for mixture-of-experts layers, one launch for all experts.  The reference has
  * no single call for it: it loops over the experts in Python and calls each expert's LowBitLinear
  * on the rows routed to it (python/llm/src/ipex_llm/transformers/models/qwen2_moe.py:375-430 is the

@@ -20,6 +20,9 @@ int launch_dequantize(const void *w, void *out, int qtype, int64_t N, int64_t K,
                       hipStream_t st);
 int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 int waves, hipStream_t st);
+size_t ring_workspace_bytes(int M, int N, int K, int wgs);
+int launch_gemm_ring(const void *x, const void *w, void *y, int qtype, int act_dtype, int M, int N, int K,
+                     void *workspace, size_t workspace_bytes, int wgs, int waves, hipStream_t st);
 int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 void *workspace, size_t workspace_bytes, int want_splits, hipStream_t st);
 int gemm_splits(int M, int N, int K, size_t ws_bytes);
@@ -138,6 +141,20 @@ int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, in
     if (K == 0) return fail(LOWBIT_ESHAPE, "lowbit_gemv: K == 0");
     return check_launch(launch_gemv(x, w, y, qtype, layout, act_dtype, (int)M, (int)N, (int)K, waves,
                                     (hipStream_t)stream), "lowbit_gemv");
+}
+
+int lowbit_gemm_ring(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
+                     int64_t K, void *workspace, size_t workspace_bytes, int wgs, int waves, void *stream) {
+    const char *what = "lowbit_gemm_ring";
+    if (int rc = check_mm(what, x, w, y, qtype, layout, act_dtype, M, N, K)) return rc;
+    if (M * N == 0) return 0;
+    if (layout != LOWBIT_LAYOUT_TILED || K < 128) return fail(LOWBIT_ESHAPE, "%s: needs the tiled layout", what);
+    if (((uintptr_t)y) & 7) return fail(LOWBIT_EARG, "%s: y must be 8-byte aligned", what);
+    if (wgs < 0 || wgs > 65535) return fail(LOWBIT_EARG, "%s: wgs must be 0 (automatic) .. 65535", what);
+    if (waves != 4 && waves != 8) return fail(LOWBIT_EARG, "%s: waves must be 4 or 8", what);
+    if (workspace && !aligned16(workspace)) return fail(LOWBIT_EARG, "%s: workspace must be 16-byte aligned", what);
+    return check_launch(launch_gemm_ring(x, w, y, qtype, act_dtype, (int)M, (int)N, (int)K, workspace,
+                                         workspace ? workspace_bytes : 0, wgs, waves, (hipStream_t)stream), what);
 }
 
 static size_t split_bytes(int64_t M, int64_t N, int splits) {

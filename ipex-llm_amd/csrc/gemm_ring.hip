@@ -1,0 +1,478 @@
+// y[M,N] = x[M,K] * dequant(W)[N,K]^T for 16 < M <= 128: a batch of decode tokens or a short prompt.
+//
+// Replaces xe_batch.batch_forward / xe_linear.forward_new at these M
+// (python/llm/src/ipex_llm/transformers/low_bit_linear.py:657-668).
+//
+// At these M the product is bound by streaming the weights once, like the GEMV, but x no longer fits
+// a wave's share of LDS, so the work is cut like a GEMM: a workgroup of 4 waves owns all rows of x
+// (32, 64 or 128 of them) by 256 weight rows and a slice of K; the slices of one tile leave fp32
+// partial sums in a workspace and a second kernel adds them (split-K fills the machine: N / 256
+// tiles alone are far fewer than CUs).
+//
+// With few workgroups per CU the memory latency is covered by depth, not by occupancy: both operands
+// of a 128-column step - the block of x and the RAW quantized tiles - travel HBM -> LDS by LDS-DMA
+// into a ring of S stages, S - 1 steps ahead of their use.  A wave fetches the weight tiles it
+// consumes itself (no barrier needed for them), the block of x is shared (one barrier per step).
+// The loads of a stage are counted, and the wait before step t leaves the loads of the younger
+// stages in flight (s_waitcnt vmcnt(n) retires loads in order).
+//
+// Bytes per launch: N*K*TS/QK of weights + x once per 256 weight rows (from L2) + partial sums;
+// HBM-bound up to M = 64, co-bound with the MFMA pipe at M = 128.
+#include "lowbit_gemm.h"
+
+namespace lowbit {
+
+constexpr int RN = 256;        // weight rows per workgroup: 16 tiles
+
+template <int QT> constexpr int ring_hdr_bytes() { return Fmt<QT>::TILE_BYTES - Fmt<QT>::TILE_CODE_BYTES; }
+// one stage: the x block in operand order [16-column step (8)][32-row block (MB)][lane (64)] x 16 B, the
+// code part of the workgroup's 16 tiles, then their header parts
+template <int QT> constexpr int ring_stage_bytes(int mb) { return mb * 8 * 1024 + 16 * Fmt<QT>::TILE_BYTES; }
+// number of stages: as many as fit 160 KB of LDS, at most 6
+template <int QT> constexpr int ring_stages(int mb) {
+    const int fit = (160 * 1024 - 64) / ring_stage_bytes<QT>(mb);
+    return fit > 6 ? 6 : fit;
+}
+
+// s_waitcnt that waits for the vector-memory counter only: vmcnt = n (6 bits, split over the
+// immediate), the export and LDS counters left at "no wait"
+template <int N> __device__ inline void wait_vm() {
+    static_assert(N >= 0 && N < 64, "vmcnt has 6 bits");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+    asm volatile("" ::: "memory");
+}
+
+// The work of a launch is the list of units u = tile * G + kt (tile = (tile_n, tile_m) pair, kt = 128-
+// column step, G = K / 128), dealt out in equal contiguous runs: workgroup b of B takes units
+// b*U/B .. (b+1)*U/B - 1.  A run may cross from one tile into the next; each piece of a tile
+// ("segment") that does not cover all of K leaves an fp32 partial tile in the workspace, in slot
+// b * seg_slots + (tile - first tile of b).
+__host__ __device__ inline int64_t ring_first_unit(int64_t b, int64_t U, int64_t B) { return b * U / B; }
+__host__ __device__ inline int64_t ring_owner(int64_t u, int64_t U, int64_t B) { return ((u + 1) * B - 1) / U; }
+
+// RNB = 32-row weight blocks per wave: 2 -> 4 waves of 64 rows, 1 -> 8 waves of 32 rows (two waves
+// per SIMD cover each other's LDS and barrier waits; x is then read from LDS by twice as many waves)
+template <int QT, typename AT, int MB, int RNB, int S>
+__global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+                                                                  AT *__restrict__ y, int M, int N, int K, int seg_slots,
+                                                                  float *__restrict__ ws) {
+    using F = Fmt<QT>;
+    using V8 = typename Vec8<AT>::type;
+    constexpr int WAVES = 8 / RNB;
+    constexpr int XB = MB * 8 * 1024, CODE = F::TILE_CODE_BYTES, HDR = ring_hdr_bytes<QT>();
+    constexpr int STAGE = ring_stage_bytes<QT>(MB);
+    constexpr int CPT = CODE / 1024;                 // 1 KiB code loads per tile
+    constexpr int TPI = 256 / HDR;                   // tiles whose headers one 256-byte load covers
+    static_assert(TPI >= 1 && TPI <= 4, "header load shape");
+    constexpr int TPW = 16 / WAVES;                  // tiles per wave
+    constexpr int XL = 8 * MB / WAVES;               // loads per stage and wave: x blocks,
+    constexpr int CL = TPW * CPT;                    //   code KiBs,
+    constexpr int HL = TPW / TPI > 0 ? TPW / TPI : 1;   // header loads (a wave with fewer tiles than a load covers repeats its neighbour's)
+    constexpr int L = XL + CL + HL;
+    static_assert((S - 2) * L < 64, "too many loads in flight for vmcnt");
+    static_assert(S >= 2 && S <= 6, "ring depth");
+    extern __shared__ __attribute__((aligned(16))) uint8_t ring[];
+    float *lut = (float *)(ring + S * STAGE);        // nf4 code book, behind the ring
+    if constexpr (QT == QT_NF4) {
+        if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODEBOOK[threadIdx.x];
+        __syncthreads();
+    }
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: LDS-DMA targets are scalars
+    const int G = K / TILE_COLS;
+    const int n_tiles = N / TILE_ROWS;
+    const int tiles_m = (M + 32 * MB - 1) / (32 * MB), tiles_n = (N + RN - 1) / RN;
+    const int kg = lane >> 5, i32 = lane & 31, r16 = lane & 15;
+    const int slot_lo = kg * 16 + r16, slot_hi = (kg + 2) * 16 + r16;
+
+    const int64_t U = (int64_t)tiles_m * tiles_n * G;
+    const int u0 = (int)ring_first_unit(blockIdx.x, U, gridDim.x), u1 = (int)ring_first_unit(blockIdx.x + 1, U, gridDim.x);
+    const int n_units = u1 - u0;
+    const int first_tile = u0 / G;
+
+    // ---- sources of this lane's share of a stage, for the tile being fetched
+    // x: one load fills the 1 KiB operand block (16-column step ks, row block mb): lane 32*kg + i
+    // fetches row 32*mb + i, columns 16*ks + 8*kg .. +7.  Wave v fills ks = v*XL/MB .. (all mb of each).
+    // weights: wave v owns tiles v*TPW .. of the workgroup's 16 (tile rows past N are clamped: they are
+    // computed and never stored).  Codes: lane l fetches bytes 16l .. of the tile (and of its second
+    // KiB for 8-bit codes).  Headers: one 4-byte load per lane, 256 bytes per instruction, which is
+    // the header part of TPI tiles.
+    gbytes xsrc[MB], csrc[TPW], hsrc[HL];
+    constexpr int HFIRST_NUM = 16 / TPI;             // header loads per stage and workgroup
+    const int hfirst = wave * HFIRST_NUM / WAVES;    // index of this wave's first header load
+    auto set_tile = [&](int tile) {
+        const int tile_m = tile % tiles_m, tile_n = tile / tiles_m;
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            int row = tile_m * 32 * MB + mb * 32 + i32;
+            row = row < M ? row : M - 1;
+            xsrc[mb] = (gbytes)x + ((int64_t)row * K + kg * 8) * (int64_t)sizeof(AT);
+        }
+#pragma unroll
+        for (int i = 0; i < TPW; i++) {
+            int trow = tile_n * 16 + wave * TPW + i;
+            trow = trow < n_tiles ? trow : n_tiles - 1;
+            csrc[i] = (gbytes)w + (int64_t)trow * G * F::TILE_BYTES + lane * 16;
+        }
+#pragma unroll
+        for (int i = 0; i < HL; i++) {
+            constexpr int LPT = 64 / TPI;            // lanes per tile
+            int trow = tile_n * 16 + (hfirst + i) * TPI + lane / LPT;
+            trow = trow < n_tiles ? trow : n_tiles - 1;
+            hsrc[i] = (gbytes)w + (int64_t)trow * G * F::TILE_BYTES + CODE + (lane % LPT) * 4;
+        }
+    };
+    const uint32_t ring_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)ring;
+
+    // Issued from inline assembly: the compiler neither counts these loads nor orders LDS accesses
+    // against them; completion is awaited by the explicit vmcnt waits below.
+    auto dma16 = [&](gbytes src, uint32_t lds) {
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
+    };
+    auto dma4 = [&](gbytes src, uint32_t lds) {
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
+    };
+    auto issue = [&](int kt, int slot) {             // exactly L loads
+        const uint32_t base = __builtin_amdgcn_readfirstlane(ring_base + slot * STAGE);
+        const int64_t xk = (int64_t)kt * TILE_COLS * sizeof(AT), wk = (int64_t)kt * F::TILE_BYTES;
+#pragma unroll
+        for (int j = 0; j < XL; j++) {
+            const int blk = wave * XL + j;           // (ks, mb) = (blk / MB, blk % MB)
+            dma16(xsrc[j % MB] + xk + (blk / MB) * 16 * sizeof(AT), base + blk * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < TPW; i++)
+#pragma unroll
+            for (int c = 0; c < CPT; c++) dma16(csrc[i] + wk + c * 1024, base + XB + (wave * TPW + i) * CODE + c * 1024);
+#pragma unroll
+        for (int i = 0; i < HL; i++) dma4(hsrc[i] + wk, base + XB + 16 * CODE + (hfirst + i) * 256);
+    };
+    static_assert(XL % MB == 0 || MB % XL == 0, "x blocks per wave");
+
+    struct WRegs {
+        TileRegs<QT> lo[RNB], hi[RNB];
+    };
+    // this lane's registers of a stage: block nb = tiles TPW*v + 2nb (rows 0-15) and TPW*v + 2nb + 1
+    auto read_w = [&](int slot, WRegs &t) {
+        const uint8_t *st = ring + slot * STAGE + XB;
+#pragma unroll
+        for (int nb = 0; nb < RNB; nb++) {
+            const int ti = wave * TPW + nb * 2 + (i32 >> 4);
+            const uint8_t *codes = st + ti * CODE;
+            const uint8_t *hdr = st + 16 * CODE + ti * HDR;
+            t.lo[nb].q0 = *(const u32x4 *)(codes + slot_lo * 16);
+            t.hi[nb].q0 = *(const u32x4 *)(codes + slot_hi * 16);
+            if constexpr (F::BITS == 8) {
+                t.lo[nb].q1 = *(const u32x4 *)(codes + 1024 + slot_lo * 16);
+                t.hi[nb].q1 = *(const u32x4 *)(codes + 1024 + slot_hi * 16);
+            }
+            if constexpr (QT == QT_SYM_INT4 || QT == QT_SYM_INT8) {
+                const u32x2 h = *(const u32x2 *)(hdr + r16 * 8);
+                t.lo[nb].h[0] = h[0]; t.lo[nb].h[1] = h[1];
+            } else if constexpr (QT == QT_ASYM_INT4) {
+                t.lo[nb].h = *(const u32x4 *)(hdr + r16 * 16);
+            } else {
+                t.lo[nb].h[0] = *(const uint32_t *)(hdr + r16 * 4);
+            }
+        }
+    };
+
+    f32x16 acc[MB][RNB];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int nb = 0; nb < RNB; nb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[mb][nb][i] = 0.0f;
+    };
+    clear_acc();
+
+    const DqCtx ctx = {lut, dq_magic<QT, AT>()};
+    auto dequant_pair = [&](const WRegs &t, int ks, int nb, int p) -> uint32_t {
+        if (ks & 1) {
+            TileRegs<QT> h = t.hi[nb];
+            h.h = t.lo[nb].h;
+            return Dequant<QT, AT>::pair(h, ks >> 1, p, ctx);
+        }
+        return Dequant<QT, AT>::pair(t.lo[nb], ks >> 1, p, ctx);
+    };
+
+    // 8 steps of 16 columns in issue order: the x operand of the next step is requested from LDS
+    // right after the MFMAs that used the current one, and the next step's weights are dequantized
+    // pair by pair between the MFMAs.
+    // The MFMAs are opaque to the compiler: should it ever copy accumulators between registers around
+    // a step, the copies must not run into an MFMA still in flight (an 8-pass MFMA needs 11 wait
+    // states before its result may be read).  All accumulators are operands, so that such copies
+    // cannot be scheduled across the statement.
+    auto acc_guard = [&]() {
+        if constexpr (MB * RNB == 1) asm volatile("s_nop 7\n\ts_nop 4" : "+a"(acc[0][0]));
+        else if constexpr (MB * RNB == 2) asm volatile("s_nop 7\n\ts_nop 4" : "+a"(acc[0][0]), "+a"(acc[MB - 1][RNB - 1]));
+        else if constexpr (MB * RNB == 4)
+            asm volatile("s_nop 7\n\ts_nop 4" : "+a"(acc[0][0]), "+a"(acc[(1 / RNB) % MB][1 % RNB]), "+a"(acc[2 / RNB][2 % RNB]),
+                         "+a"(acc[3 / RNB][3 % RNB]));
+        else
+            asm volatile("s_nop 7\n\ts_nop 4" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[1][0]), "+a"(acc[1][1]),
+                         "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[3][0]), "+a"(acc[3][1]));
+    };
+    auto compute = [&](const uint8_t *cur, const WRegs &t) {
+        constexpr int PER = 4 / MB;                  // dequantized pairs per MFMA slot
+        V8 xv[MB];
+        u32x4 wv[RNB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) xv[mb] = *(const V8 *)(cur + mb * 1024 + lane * 16);
+#pragma unroll
+        for (int nb = 0; nb < RNB; nb++)
+#pragma unroll
+            for (int p = 0; p < 4; p++) wv[nb][p] = dequant_pair(t, 0, nb, p);
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            u32x4 wn[RNB];
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+#pragma unroll
+                for (int nb = 0; nb < RNB; nb++) {
+                    mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    if (ks < 7) {
+#pragma unroll
+                        for (int q = 0; q < PER; q++) {
+                            const int idx = (mb * RNB + nb) * PER + q;
+                            wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);
+                        }
+                    }
+                }
+                if (ks < 7) xv[mb] = *(const V8 *)(cur + ((ks + 1) * MB + mb) * 1024 + lane * 16);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (ks < 7) {
+#pragma unroll
+                for (int nb = 0; nb < RNB; nb++) wv[nb] = wn[nb];
+            }
+        }
+        acc_guard();
+    };
+
+    // Writes the finished segment of `tile`: straight to y when it covers all of K, else as a partial
+    // tile.  C layout of a 32x32 block: lane = 32*g + column (= row of x), register i = weight row
+    // 8*(i/4) + 4*g + i%4.
+    auto store_segment = [&](int tile, bool whole) {
+        // The MFMAs are opaque to the compiler's hazard tracking: the accumulators are operands of
+        // the wait statement so that no read of them can be scheduled ahead of it.
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int nb = 0; nb < RNB; nb++)
+                asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7" : "+a"(acc[mb][nb]));
+        const int m0 = (tile % tiles_m) * 32 * MB, n0 = (tile / tiles_m) * RN + wave * (32 * RNB);
+        // partial sums keep the register layout (slot, wave, register group, lane): every store
+        // instruction writes 1 KiB contiguous
+        float *part = ws + ((int64_t)blockIdx.x * seg_slots + (tile - first_tile)) * (32 * MB * RN);
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            const int m = m0 + mb * 32 + i32;
+            if (m < M) {
+#pragma unroll
+                for (int nb = 0; nb < RNB; nb++) {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const int n = n0 + nb * 32 + q * 8 + kg * 4;
+                        if (n < N) {
+                            if (!whole) {
+                                const f32x4 o = {acc[mb][nb][q * 4], acc[mb][nb][q * 4 + 1], acc[mb][nb][q * 4 + 2],
+                                                 acc[mb][nb][q * 4 + 3]};
+                                const int grp = (mb * RNB + nb) * 4 + q;
+                                *(f32x4 *)(part + ((wave * (MB * RNB * 4) + grp) * 64 + lane) * 4) = o;
+                            } else {
+                                typedef AT at4 __attribute__((ext_vector_type(4)));
+                                at4 o;
+#pragma unroll
+                                for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
+                                *(at4 *)(y + (int64_t)m * N + n) = o;
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    };
+
+    // ---- the ring.  The i-th unit of this workgroup lives in slot i % S.  Before unit i is used, the
+    // units i+1 .. min(n, i+S-1)-1 may still be in flight; everything older has to have landed.
+    auto wait_for = [&](int younger) {              // number of whole stages that may stay in flight
+        switch (younger) {
+        case 0: wait_vm<0>(); break;
+        case 1: wait_vm<(S > 2 ? 1 : 0) * L>(); break;
+        case 2: wait_vm<(S > 3 ? 2 : 0) * L>(); break;
+        case 3: wait_vm<(S > 4 ? 3 : 0) * L>(); break;
+        default: wait_vm<(S > 5 ? 4 : 0) * L>(); break;
+        }
+    };
+    int f_tile = first_tile, f_kt = u0 - first_tile * G;      // fetch position
+    set_tile(f_tile);
+    auto issue_next = [&](int slot) {
+        issue(f_kt, slot);
+        if (++f_kt == G) {
+            f_kt = 0;
+            f_tile++;
+            set_tile(f_tile);                        // one tile past the end at worst: clamped, never fetched
+        }
+    };
+#pragma unroll
+    for (int s = 0; s < S - 1; s++)
+        if (s < n_units) issue_next(s);
+    int slot = 0, fill = S - 1;                      // slot of the current unit / of the next one to fill
+    int c_tile = first_tile, c_kt = u0 - first_tile * G;
+    WRegs wr;
+    // one pass of the outer loop per segment, so that the accumulators are loop-carried by the inner
+    // loop only and stay where the MFMAs want them
+    for (int i = 0; i < n_units;) {
+        const int seg_len = n_units - i < G - c_kt ? n_units - i : G - c_kt;
+        const int seg_end = i + seg_len;
+        clear_acc();
+        for (; i < seg_end; i++) {
+            const int issued = n_units < i + S - 1 ? n_units : i + S - 1;
+            wait_for(issued - i - 1);
+            // every wave's part of x for this stage has landed, and every wave is done with the
+            // previous stage, whose slot is the one refilled next
+            __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0): this wave's LDS reads of the previous stage are done
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (i + S - 1 < n_units) issue_next(fill);
+            read_w(slot, wr);
+            compute(ring + slot * STAGE, wr);
+            slot = slot + 1 == S ? 0 : slot + 1;
+            fill = fill + 1 == S ? 0 : fill + 1;
+        }
+        store_segment(c_tile, seg_len == G);
+        c_tile++;
+        c_kt = 0;
+    }
+}
+
+// Sums the partial tiles of every output tile that was cut into segments and writes y, rounded once.
+// One thread per group of 4 consecutive n, in the order the partial sums were stored.
+template <typename AT, int MB, int RNB>
+__global__ __launch_bounds__(256) void ring_reduce_kernel(const float *__restrict__ ws, AT *__restrict__ y, int M, int N,
+                                                          int G, int tiles, int B, int seg_slots) {
+    constexpr int WAVES = 8 / RNB, GRP = MB * RNB * 4;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;       // (tile, wave, group, lane)
+    if (t >= (int64_t)tiles * WAVES * GRP * 64) return;
+    const int lane = (int)(t & 63);
+    const int grp = (int)((t >> 6) % GRP);
+    const int wave = (int)((t >> 6) / GRP % WAVES);
+    const int tile = (int)((t >> 6) / GRP / WAVES);
+    const int tiles_m = (M + 32 * MB - 1) / (32 * MB);
+    const int mb = grp / (RNB * 4), nb = grp / 4 % RNB, q = grp % 4;
+    const int m = (tile % tiles_m) * 32 * MB + mb * 32 + (lane & 31);
+    const int n = (tile / tiles_m) * RN + wave * (32 * RNB) + nb * 32 + q * 8 + (lane >> 5) * 4;
+    if (m >= M || n >= N) return;
+    const int64_t U = (int64_t)tiles * G;
+    const int b0 = (int)ring_owner((int64_t)tile * G, U, B), b1 = (int)ring_owner((int64_t)(tile + 1) * G - 1, U, B);
+    if (b0 == b1) return;                            // one segment covered all of K and wrote y itself
+    f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int b = b0; b <= b1; b++) {
+        const int seg = tile - (int)(ring_first_unit(b, U, B) / G);
+        const float *part = ws + ((int64_t)b * seg_slots + seg) * (32 * MB * RN);
+        a += *(const f32x4 *)(part + ((wave * GRP + grp) * 64 + lane) * 4);
+    }
+    typedef AT at4 __attribute__((ext_vector_type(4)));
+    at4 o;
+#pragma unroll
+    for (int k = 0; k < 4; k++) o[k] = to_at<AT>(a[k]);
+    *(at4 *)(y + (int64_t)m * N + n) = o;
+}
+
+struct RingPlan {
+    int mb, tiles, B, seg_slots;
+    size_t ws_bytes;
+};
+
+// wgs = number of workgroups to deal the units to (0: one per CU, never fewer than one per two units);
+// without a workspace every workgroup takes whole tiles
+static RingPlan ring_plan(int M, int N, int K, int wgs, bool have_ws) {
+    RingPlan p;
+    p.mb = M <= 32 ? 1 : M <= 64 ? 2 : 4;
+    p.tiles = ((M + 32 * p.mb - 1) / (32 * p.mb)) * ((N + RN - 1) / RN);
+    const int G = K / TILE_COLS;
+    const int64_t U = (int64_t)p.tiles * G;
+    int64_t B = wgs > 0 ? wgs : 256;
+    if (B > U / 2) B = U / 2 > 0 ? U / 2 : 1;
+    if (!have_ws || B <= p.tiles) {
+        // whole tiles only
+        B = B < p.tiles ? B : p.tiles;
+        if (!have_ws) B = p.tiles;
+    }
+    p.B = (int)B;
+    // a run of ceil(U/B) units touches at most this many tiles
+    const int64_t run = (U + B - 1) / B;
+    p.seg_slots = (int)((run + G - 2) / G) + 1;
+    p.ws_bytes = (U % B == 0 && (U / B) % G == 0) ? 0 : (size_t)B * p.seg_slots * (32 * p.mb) * RN * sizeof(float);
+    return p;
+}
+
+size_t ring_workspace_bytes(int M, int N, int K, int wgs) { return ring_plan(M, N, K, wgs, true).ws_bytes; }
+
+template <int QT, typename AT, int MB, int RNB>
+static int launch_ring_m(const void *x, const void *w, void *y, int M, int N, int K, float *ws, const RingPlan &p,
+                         hipStream_t st) {
+    constexpr int S = ring_stages<QT>(MB);
+    constexpr int LDS = S * ring_stage_bytes<QT>(MB) + 64;
+    auto kern = gemm_ring_kernel<QT, AT, MB, RNB, S>;
+    static bool raised = false;                      // the default limit of dynamic LDS is 64 KB
+    if (!raised) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) return -6;
+        raised = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(p.B), dim3(512 / RNB), LDS, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K,
+                       p.seg_slots, ws);
+    if (p.ws_bytes) {
+        const int64_t threads = (int64_t)p.tiles * (32 * MB) * RN / 4;
+        hipLaunchKernelGGL((ring_reduce_kernel<AT, MB, RNB>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, ws,
+                           (AT *)y, M, N, K / TILE_COLS, p.tiles, p.B, p.seg_slots);
+    }
+    return 0;
+}
+
+template <int QT, typename AT>
+static int launch_ring_t(const void *x, const void *w, void *y, int M, int N, int K, float *ws, const RingPlan &p,
+                         int waves, hipStream_t st) {
+    if (waves == 4) {
+        if (p.mb == 1) return launch_ring_m<QT, AT, 1, 2>(x, w, y, M, N, K, ws, p, st);
+        if (p.mb == 2) return launch_ring_m<QT, AT, 2, 2>(x, w, y, M, N, K, ws, p, st);
+        return launch_ring_m<QT, AT, 4, 2>(x, w, y, M, N, K, ws, p, st);
+    }
+    if (p.mb == 1) return launch_ring_m<QT, AT, 1, 1>(x, w, y, M, N, K, ws, p, st);
+    if (p.mb == 2) return launch_ring_m<QT, AT, 2, 1>(x, w, y, M, N, K, ws, p, st);
+    return launch_ring_m<QT, AT, 4, 1>(x, w, y, M, N, K, ws, p, st);
+}
+
+template <int QT>
+static int launch_ring_q(const void *x, const void *w, void *y, int dt, int M, int N, int K, float *ws, const RingPlan &p,
+                         int waves, hipStream_t st) {
+    if (dt == DT_F16) return launch_ring_t<QT, _Float16>(x, w, y, M, N, K, ws, p, waves, st);
+    if (dt == DT_BF16) return launch_ring_t<QT, __bf16>(x, w, y, M, N, K, ws, p, waves, st);
+    return -4;
+}
+
+// Tiled layout only; the caller has checked the shape and the alignment of y (8 bytes).  A workspace
+// smaller than ring_workspace_bytes() for the same `wgs` is not used: the tiles are then not cut.
+int launch_gemm_ring(const void *x, const void *w, void *y, int qtype, int act_dtype, int M, int N, int K,
+                     void *workspace, size_t workspace_bytes, int wgs, int waves, hipStream_t st) {
+    if (M == 0 || N == 0) return 0;
+    RingPlan p = ring_plan(M, N, K, wgs, workspace != nullptr);
+    if (p.ws_bytes > workspace_bytes) p = ring_plan(M, N, K, wgs, false);
+    float *ws = (float *)workspace;
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_ring_q<QT_SYM_INT4>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
+    case QT_ASYM_INT4: return launch_ring_q<QT_ASYM_INT4>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
+    case QT_SYM_INT8: return launch_ring_q<QT_SYM_INT8>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
+    case QT_NF4: return launch_ring_q<QT_NF4>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
+    case QT_FP8_E4M3: return launch_ring_q<QT_FP8_E4M3>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
+    default: return -2;
+    }
+}
+
+}  // namespace lowbit

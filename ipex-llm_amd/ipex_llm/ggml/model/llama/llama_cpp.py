@@ -184,6 +184,9 @@ _lib.lowbit_forward_ws.restype = c_int
 _lib.lowbit_gemm_ws.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
                                 c_void_p, c_size_t, c_int, c_void_p]
 _lib.lowbit_gemm_ws.restype = c_int
+_lib.lowbit_gemm_ring.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
+                                  c_void_p, c_size_t, c_int, c_int, c_void_p]
+_lib.lowbit_gemm_ring.restype = c_int
 
 
 def lowbit_workspace_bytes(m, n, k) -> int:
@@ -198,6 +201,11 @@ def lowbit_forward_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, wor
 def lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, splits, stream):
     _check(_lib.lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, splits, stream),
            "lowbit_gemm_ws")
+
+
+def lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, wgs, waves, stream):
+    _check(_lib.lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, wgs, waves,
+                                 stream), "lowbit_gemm_ring")
 
 
 _lib.lowbit_grouped_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int,
