@@ -53,6 +53,8 @@ def main():
                     help="run only the serialized [11008 x 4096] GEMV loop the roofline object is measured on")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the prefill GEMM (M=2048 on [11008 x 4096], sym_int4, fp16) and print its rate")
+    ap.add_argument("--batch-only", action="store_true",
+                    help="run only the batch-sized product (M=32, 64, 128 on [11008 x 4096], sym_int4, fp16)")
     ap.add_argument("--quantize-only", action="store_true",
                     help="run only the block quantizer (fp32 [11008 x 4096] -> sym_int4, tiled) and print its rate")
     args = ap.parse_args()
@@ -206,6 +208,33 @@ def main():
 
     if args.prefill_only:
         print(json.dumps({"prefill": prefill_leg()}))
+        return
+
+    def batch_leg(m):
+        """One [11008 x 4096] linear at a serving batch of M rows, cycling over the 64 distinct gate / up
+        weights (1.6 GB, far beyond the Infinity Cache) per graph replay, with the workspace the library
+        asks for (HBM-bound: the weights are read once)."""
+        gu8 = [b for mods in layers for (name, n, k, b) in mods if name in ("gate", "up")]
+        xp = torch.randn((m, 4096), generator=gen, device=dev, dtype=torch.float32).half()
+        yp = torch.empty((m, 11008), dtype=torch.float16, device=dev)
+        ws_bytes = max(16, ggml.lowbit_workspace_bytes(m, 11008, 4096))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+        def batch():
+            st = stream()
+            for b in gu8:
+                ggml.lowbit_forward_ws(xp.data_ptr(), b.data_ptr(), yp.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED,
+                                       ggml.DT_F16, m, 11008, 4096, ws.data_ptr(), ws_bytes, st)
+        gb = capture(batch)
+        msb = time_graph(gb, 5, 3) / len(gu8)
+        hb = blob_bytes(11008, 4096) + m * 4096 * 2 + m * 11008 * 2
+        return {"kernel": "gemm_ring_kernel<sym_int4,f16> + reduction on [11008 x 4096], M=%d" % m, "bound": "hbm",
+                "bytes_per_launch": hb, "ms": round(msb, 4), "achieved": round(hb / (msb * 1e-3) / 1e9, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(hb / (msb * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "TFLOP/s": round(2.0 * m * 11008 * 4096 / (msb * 1e-3) / 1e12, 1)}
+
+    if args.batch_only:
+        print(json.dumps({"batch": {"M%d" % m: batch_leg(m) for m in (32, 64, 128)}}))
         return
 
     # ---- roofline leg: the metric's single shape (N=11008, K=4096) as a serialized chain of
@@ -371,6 +400,9 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream):
     for name, mods in (("sym_int4", sym), ("asym_int4", asym)):
         for m in (512, 2048):
             res[f"prefill_layer_{name}_M{m}"] = time_set(mods, QT[name], ggml.DT_F16, torch.float16, m, 5)
+    # the same layer at serving batch sizes (one decode token per sequence)
+    for m in (32, 64, 128):
+        res[f"batched_decode_layer_sym_int4_M{m}"] = time_set(sym, QT["sym_int4"], ggml.DT_F16, torch.float16, m, 10)
     del asym
     # configs[3]: Llama-3-70B linear set (q, k, v, gate, up, down), bf16
     shapes70 = [(8192, 8192), (1024, 8192), (1024, 8192), (28672, 8192), (28672, 8192), (8192, 28672)]

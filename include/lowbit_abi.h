@@ -159,8 +159,12 @@ int lowbit_forward_ws(const void *x, const void *w, void *y, int qtype, int layo
 int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
                    int64_t K, void *workspace, size_t workspace_bytes, int splits, void *stream);
 
+/* The kernel lowbit_forward_ws picks for M of a few dozen to a few hundred rows (tiled layout, y
+ * 8-byte aligned): 128 / 64 / 32 rows of x by 256 weight rows per workgroup, the (tile, K-step) units
+ * dealt out in equal runs over `wgs` workgroups (0 = the library's choice), partial tiles summed from
+ * the workspace.  A null or too small workspace is valid: tiles are then not cut along K. */
 int lowbit_gemm_ring(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
-                     int64_t K, void *workspace, size_t workspace_bytes, int wgs, int waves, void *stream);
+                     int64_t K, void *workspace, size_t workspace_bytes, int wgs, void *stream);
 
 /* Grouped product for mixture-of-experts layers, one launch for all experts.  The reference has
  * no single call for it: it loops over the experts in Python and calls each expert's LowBitLinear

@@ -21,8 +21,9 @@ int launch_dequantize(const void *w, void *out, int qtype, int64_t N, int64_t K,
 int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 int waves, hipStream_t st);
 size_t ring_workspace_bytes(int M, int N, int K, int wgs);
+double ring_time_us(int M, int N, int K, int qtype, bool have_ws);
 int launch_gemm_ring(const void *x, const void *w, void *y, int qtype, int act_dtype, int M, int N, int K,
-                     void *workspace, size_t workspace_bytes, int wgs, int waves, hipStream_t st);
+                     void *workspace, size_t workspace_bytes, int wgs, hipStream_t st);
 int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 void *workspace, size_t workspace_bytes, int want_splits, hipStream_t st);
 int gemm_splits(int M, int N, int K, size_t ws_bytes);
@@ -144,17 +145,16 @@ int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, in
 }
 
 int lowbit_gemm_ring(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
-                     int64_t K, void *workspace, size_t workspace_bytes, int wgs, int waves, void *stream) {
+                     int64_t K, void *workspace, size_t workspace_bytes, int wgs, void *stream) {
     const char *what = "lowbit_gemm_ring";
     if (int rc = check_mm(what, x, w, y, qtype, layout, act_dtype, M, N, K)) return rc;
     if (M * N == 0) return 0;
     if (layout != LOWBIT_LAYOUT_TILED || K < 128) return fail(LOWBIT_ESHAPE, "%s: needs the tiled layout", what);
     if (((uintptr_t)y) & 7) return fail(LOWBIT_EARG, "%s: y must be 8-byte aligned", what);
     if (wgs < 0 || wgs > 65535) return fail(LOWBIT_EARG, "%s: wgs must be 0 (automatic) .. 65535", what);
-    if (waves != 4 && waves != 8) return fail(LOWBIT_EARG, "%s: waves must be 4 or 8", what);
     if (workspace && !aligned16(workspace)) return fail(LOWBIT_EARG, "%s: workspace must be 16-byte aligned", what);
     return check_launch(launch_gemm_ring(x, w, y, qtype, act_dtype, (int)M, (int)N, (int)K, workspace,
-                                         workspace ? workspace_bytes : 0, wgs, waves, (hipStream_t)stream), what);
+                                         workspace ? workspace_bytes : 0, wgs, (hipStream_t)stream), what);
 }
 
 static size_t split_bytes(int64_t M, int64_t N, int splits) {
@@ -192,9 +192,13 @@ int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout,
 }
 
 size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    if (M <= 16 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;   // M <= 16: GEMV
+    if (M <= 16 || N <= 0 || K < 128 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;   // M <= 16: GEMV
+    if (N % 16 || K % 128) return 0;                                                                  // not tileable: GEMV
+    // enough for whichever kernel lowbit_forward_ws may pick for the shape
     const int s = gemm_splits((int)M, (int)N, (int)K, (size_t)-1);
-    return s > 1 ? split_bytes(M, N, s) : 0;
+    const size_t gemm = s > 1 ? split_bytes(M, N, s) : 0;
+    const size_t ring = M <= 512 ? ring_workspace_bytes((int)M, (int)N, (int)K, 0) : 0;
+    return gemm > ring ? gemm : ring;
 }
 
 // Choice of kernel behind lowbit_forward, by estimated run time (constants measured on MI355X).  The
@@ -202,7 +206,8 @@ size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 // partly out of the Infinity Cache).  The MFMA GEMM amortizes the dequantization over 128 x 256 tiles
 // but is latency-bound while its tiles do not fill the machine: a lone row tile of [11008 x 4096] takes
 // 61 us however few rows it holds, where a GEMV pass takes 12 us.  With a workspace the GEMM can split
-// K over more workgroups at the price of writing and re-reading fp32 partial sums.
+// K over more workgroups at the price of writing and re-reading fp32 partial sums, and the ring kernel
+// (32 / 64 / 128-row tiles, units dealt out evenly) covers the batch sizes in between.
 static int forward_any(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
                        int64_t N, int64_t K, void *workspace, size_t workspace_bytes, void *stream) {
     if (M <= 16 || layout != LOWBIT_LAYOUT_TILED)
@@ -210,9 +215,21 @@ static int forward_any(const void *x, const void *w, void *y, int qtype, int lay
     if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || K < 128)
         return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);     // reports the error
     const double passes = (double)((M + 15) / 16);
-    const double t_gemv = passes * ((double)lowbit_blob_bytes(qtype, N * K) / 2.8e6 + 2.5);
+    // a pass cannot be shorter than its workgroups' walk along K (narrow weights leave CUs idle)
+    const double stream_us = (double)lowbit_blob_bytes(qtype, N * K) / 2.8e6, walk_us = 0.07 * (double)(K / 128);
+    const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
     const int splits = workspace ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
     const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits);
+    // The ring kernel (M up to a few hundred rows, y 8-byte aligned) needs the workspace for its partial
+    // tiles; given that, it measured faster than the tiled GEMM, split or not, up to about 7e10 FLOP
+    // (sym_int4 and sym_int8, seven shapes from [1024 x 8192] to [28672 x 8192], M = 24 .. 512), and
+    // its own estimate decides against the GEMV.
+    if (M <= 512 && !(((uintptr_t)y) & 7) && workspace && (double)M * (double)N * (double)K < 3.5e10 &&
+        ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes) {
+        if (ring_time_us((int)M, (int)N, (int)K, qtype, true) < t_gemv)
+            return lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, 0, stream);
+        return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
+    }
     if (t_gemv < t_gemm) return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
     if (splits > 1)
         return lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, splits, stream);

@@ -1,23 +1,23 @@
-// y[M,N] = x[M,K] * dequant(W)[N,K]^T for 16 < M <= 128: a batch of decode tokens or a short prompt.
+// y[M,N] = x[M,K] * dequant(W)[N,K]^T for M of a few dozen to a few hundred rows: a batch of decode
+// tokens or a short prompt.
 //
 // Replaces xe_batch.batch_forward / xe_linear.forward_new at these M
 // (python/llm/src/ipex_llm/transformers/low_bit_linear.py:657-668).
 //
 // At these M the product is bound by streaming the weights once, like the GEMV, but x no longer fits
-// a wave's share of LDS, so the work is cut like a GEMM: a workgroup of 4 waves owns all rows of x
-// (32, 64 or 128 of them) by 256 weight rows and a slice of K; the slices of one tile leave fp32
-// partial sums in a workspace and a second kernel adds them (split-K fills the machine: N / 256
-// tiles alone are far fewer than CUs).
+// a wave's share of LDS, so the work is cut like a GEMM: a workgroup of 8 waves owns 32, 64 or 128
+// rows of x by 256 weight rows (32 per wave).  N / 256 tiles are far fewer than CUs, so K is cut
+// as well: the list of (tile, 128-column step) units is dealt out in equal contiguous runs, one per
+// workgroup, whatever the shape; a run that covers only part of a tile's K leaves an fp32 partial
+// tile in a workspace and a second kernel adds the parts.
 //
-// With few workgroups per CU the memory latency is covered by depth, not by occupancy: both operands
-// of a 128-column step - the block of x and the RAW quantized tiles - travel HBM -> LDS by LDS-DMA
-// into a ring of S stages, S - 1 steps ahead of their use.  A wave fetches the weight tiles it
-// consumes itself (no barrier needed for them), the block of x is shared (one barrier per step).
-// The loads of a stage are counted, and the wait before step t leaves the loads of the younger
-// stages in flight (s_waitcnt vmcnt(n) retires loads in order).
+// Both operands of a step - the block of x and the RAW quantized tiles - travel HBM -> LDS by
+// LDS-DMA into a ring of stages, ahead of their use.  A wave fetches the weight tiles it consumes
+// itself (no barrier needed for them), the block of x is shared (one barrier per step).  The loads
+// of a stage are counted, and the wait before a step leaves the loads of the younger stages in
+// flight (s_waitcnt vmcnt(n) retires loads in order).
 //
-// Bytes per launch: N*K*TS/QK of weights + x once per 256 weight rows (from L2) + partial sums;
-// HBM-bound up to M = 64, co-bound with the MFMA pipe at M = 128.
+// Bytes per launch: N*K*TS/QK of weights + x once per 256 weight rows (from L2) + partial sums.
 #include "lowbit_gemm.h"
 
 namespace lowbit {
@@ -28,10 +28,11 @@ template <int QT> constexpr int ring_hdr_bytes() { return Fmt<QT>::TILE_BYTES - 
 // one stage: the x block in operand order [16-column step (8)][32-row block (MB)][lane (64)] x 16 B, the
 // code part of the workgroup's 16 tiles, then their header parts
 template <int QT> constexpr int ring_stage_bytes(int mb) { return mb * 8 * 1024 + 16 * Fmt<QT>::TILE_BYTES; }
-// number of stages: as many as fit 160 KB of LDS, at most 6
+// number of stages: 3, or 2 where 3 do not fit 160 KB of LDS.  A deeper ring measured no faster: the
+// loads that a CU can keep in flight are bounded elsewhere.
 template <int QT> constexpr int ring_stages(int mb) {
     const int fit = (160 * 1024 - 64) / ring_stage_bytes<QT>(mb);
-    return fit > 6 ? 6 : fit;
+    return fit > 3 ? 3 : fit;
 }
 
 // s_waitcnt that waits for the vector-memory counter only: vmcnt = n (6 bits, split over the
@@ -218,10 +219,12 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
     };
     auto compute = [&](const uint8_t *cur, const WRegs &t) {
         constexpr int PER = 4 / MB;                  // dequantized pairs per MFMA slot
-        V8 xv[MB];
+        V8 xv[2][MB];                                // x operands of this 16-column step and the next
         u32x4 wv[RNB];
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) xv[mb] = *(const V8 *)(cur + mb * 1024 + lane * 16);
+        for (int k = 0; k < 2; k++)
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) xv[k][mb] = *(const V8 *)(cur + (k * MB + mb) * 1024 + lane * 16);
 #pragma unroll
         for (int nb = 0; nb < RNB; nb++)
 #pragma unroll
@@ -233,7 +236,7 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
             for (int mb = 0; mb < MB; mb++) {
 #pragma unroll
                 for (int nb = 0; nb < RNB; nb++) {
-                    mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[ks & 1][mb]);
                     if (ks < 7) {
 #pragma unroll
                         for (int q = 0; q < PER; q++) {
@@ -242,7 +245,8 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
                         }
                     }
                 }
-                if (ks < 7) xv[mb] = *(const V8 *)(cur + ((ks + 1) * MB + mb) * 1024 + lane * 16);
+                // two steps ahead: one MFMA slot is shorter than the LDS latency when MB is small
+                if (ks < 6) xv[ks & 1][mb] = *(const V8 *)(cur + ((ks + 2) * MB + mb) * 1024 + lane * 16);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (ks < 7) {
@@ -390,27 +394,39 @@ struct RingPlan {
     size_t ws_bytes;
 };
 
-// wgs = number of workgroups to deal the units to (0: one per CU, never fewer than one per two units);
-// without a workspace every workgroup takes whole tiles
+// wgs = number of workgroups to deal the units to; 0 = one per CU, but at least four units each (the
+// fixed cost of a workgroup and its partial tile are not worth less).  Without a workspace every
+// workgroup takes whole tiles.
 static RingPlan ring_plan(int M, int N, int K, int wgs, bool have_ws) {
     RingPlan p;
     p.mb = M <= 32 ? 1 : M <= 64 ? 2 : 4;
     p.tiles = ((M + 32 * p.mb - 1) / (32 * p.mb)) * ((N + RN - 1) / RN);
     const int G = K / TILE_COLS;
     const int64_t U = (int64_t)p.tiles * G;
-    int64_t B = wgs > 0 ? wgs : 256;
-    if (B > U / 2) B = U / 2 > 0 ? U / 2 : 1;
-    if (!have_ws || B <= p.tiles) {
-        // whole tiles only
-        B = B < p.tiles ? B : p.tiles;
-        if (!have_ws) B = p.tiles;
-    }
+    int64_t B = wgs > 0 ? wgs : (U / 4 < 256 ? U / 4 : 256);
+    if (B > U) B = U;
+    if (B < 1) B = 1;
+    if (!have_ws) B = p.tiles;
     p.B = (int)B;
     // a run of ceil(U/B) units touches at most this many tiles
     const int64_t run = (U + B - 1) / B;
     p.seg_slots = (int)((run + G - 2) / G) + 1;
     p.ws_bytes = (U % B == 0 && (U / B) % G == 0) ? 0 : (size_t)B * p.seg_slots * (32 * p.mb) * RN * sizeof(float);
     return p;
+}
+
+// Estimated run time in microseconds, from measurements on MI355X (sym_int4, fp16): a fixed part
+// (launch, first loads, partial tiles and their reduction) plus the steps of the longest run; 8-bit
+// codes measured 10% slower.
+double ring_time_us(int M, int N, int K, int qtype, bool have_ws) {
+    const RingPlan p = ring_plan(M, N, K, 0, have_ws);
+    static const double fixed[3] = {11.3, 13.1, 17.3}, step[3] = {1.12, 1.55, 2.56};
+    const int i = p.mb == 1 ? 0 : p.mb == 2 ? 1 : 2;
+    const int64_t U = (int64_t)p.tiles * (K / TILE_COLS);
+    const double run = (double)((U + p.B - 1) / p.B);
+    const double bytes = (qtype == QT_SYM_INT8 || qtype == QT_FP8_E4M3) ? 1.1 : 1.0;
+    const double busy = p.B >= 256 ? 1.0 : 0.8 + 0.2 * p.B / 256.0;     // steps are shorter on a machine that is not full
+    return fixed[i] - (p.ws_bytes ? 0.0 : 4.5) + run * step[i] * bytes * busy;
 }
 
 size_t ring_workspace_bytes(int M, int N, int K, int wgs) { return ring_plan(M, N, K, wgs, true).ws_bytes; }
@@ -438,12 +454,7 @@ static int launch_ring_m(const void *x, const void *w, void *y, int M, int N, in
 
 template <int QT, typename AT>
 static int launch_ring_t(const void *x, const void *w, void *y, int M, int N, int K, float *ws, const RingPlan &p,
-                         int waves, hipStream_t st) {
-    if (waves == 4) {
-        if (p.mb == 1) return launch_ring_m<QT, AT, 1, 2>(x, w, y, M, N, K, ws, p, st);
-        if (p.mb == 2) return launch_ring_m<QT, AT, 2, 2>(x, w, y, M, N, K, ws, p, st);
-        return launch_ring_m<QT, AT, 4, 2>(x, w, y, M, N, K, ws, p, st);
-    }
+                         hipStream_t st) {
     if (p.mb == 1) return launch_ring_m<QT, AT, 1, 1>(x, w, y, M, N, K, ws, p, st);
     if (p.mb == 2) return launch_ring_m<QT, AT, 2, 1>(x, w, y, M, N, K, ws, p, st);
     return launch_ring_m<QT, AT, 4, 1>(x, w, y, M, N, K, ws, p, st);
@@ -451,26 +462,26 @@ static int launch_ring_t(const void *x, const void *w, void *y, int M, int N, in
 
 template <int QT>
 static int launch_ring_q(const void *x, const void *w, void *y, int dt, int M, int N, int K, float *ws, const RingPlan &p,
-                         int waves, hipStream_t st) {
-    if (dt == DT_F16) return launch_ring_t<QT, _Float16>(x, w, y, M, N, K, ws, p, waves, st);
-    if (dt == DT_BF16) return launch_ring_t<QT, __bf16>(x, w, y, M, N, K, ws, p, waves, st);
+                         hipStream_t st) {
+    if (dt == DT_F16) return launch_ring_t<QT, _Float16>(x, w, y, M, N, K, ws, p, st);
+    if (dt == DT_BF16) return launch_ring_t<QT, __bf16>(x, w, y, M, N, K, ws, p, st);
     return -4;
 }
 
 // Tiled layout only; the caller has checked the shape and the alignment of y (8 bytes).  A workspace
 // smaller than ring_workspace_bytes() for the same `wgs` is not used: the tiles are then not cut.
 int launch_gemm_ring(const void *x, const void *w, void *y, int qtype, int act_dtype, int M, int N, int K,
-                     void *workspace, size_t workspace_bytes, int wgs, int waves, hipStream_t st) {
+                     void *workspace, size_t workspace_bytes, int wgs, hipStream_t st) {
     if (M == 0 || N == 0) return 0;
     RingPlan p = ring_plan(M, N, K, wgs, workspace != nullptr);
     if (p.ws_bytes > workspace_bytes) p = ring_plan(M, N, K, wgs, false);
     float *ws = (float *)workspace;
     switch (qtype) {
-    case QT_SYM_INT4: return launch_ring_q<QT_SYM_INT4>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
-    case QT_ASYM_INT4: return launch_ring_q<QT_ASYM_INT4>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
-    case QT_SYM_INT8: return launch_ring_q<QT_SYM_INT8>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
-    case QT_NF4: return launch_ring_q<QT_NF4>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
-    case QT_FP8_E4M3: return launch_ring_q<QT_FP8_E4M3>(x, w, y, act_dtype, M, N, K, ws, p, waves, st);
+    case QT_SYM_INT4: return launch_ring_q<QT_SYM_INT4>(x, w, y, act_dtype, M, N, K, ws, p, st);
+    case QT_ASYM_INT4: return launch_ring_q<QT_ASYM_INT4>(x, w, y, act_dtype, M, N, K, ws, p, st);
+    case QT_SYM_INT8: return launch_ring_q<QT_SYM_INT8>(x, w, y, act_dtype, M, N, K, ws, p, st);
+    case QT_NF4: return launch_ring_q<QT_NF4>(x, w, y, act_dtype, M, N, K, ws, p, st);
+    case QT_FP8_E4M3: return launch_ring_q<QT_FP8_E4M3>(x, w, y, act_dtype, M, N, K, ws, p, st);
     default: return -2;
     }
 }

@@ -185,7 +185,7 @@ _lib.lowbit_gemm_ws.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_in
                                 c_void_p, c_size_t, c_int, c_void_p]
 _lib.lowbit_gemm_ws.restype = c_int
 _lib.lowbit_gemm_ring.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
-                                  c_void_p, c_size_t, c_int, c_int, c_void_p]
+                                  c_void_p, c_size_t, c_int, c_void_p]
 _lib.lowbit_gemm_ring.restype = c_int
 
 
@@ -203,8 +203,8 @@ def lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, worksp
            "lowbit_gemm_ws")
 
 
-def lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, wgs, waves, stream):
-    _check(_lib.lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, wgs, waves,
+def lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, wgs, stream):
+    _check(_lib.lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, wgs,
                                  stream), "lowbit_gemm_ring")
 
 

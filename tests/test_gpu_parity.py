@@ -323,6 +323,6 @@ def test_split_k_gemm_against_oracle(qtype, dtype, m, n, k, splits):
 def test_workspace_query_is_consistent():
     for m, n, k in [(256, 4096, 11008), (64, 28672, 8192), (2048, 11008, 4096), (8, 4096, 4096)]:
         b = ggml.lowbit_workspace_bytes(m, n, k)
-        assert b % (128 * 256 * 4) == 0
+        assert b % (32 * 256 * 4) == 0                              # whole partial tiles of either kernel
     assert ggml.lowbit_workspace_bytes(256, 4096, 11008) > 0        # 32 tiles, 86 steps: worth splitting
     assert ggml.lowbit_workspace_bytes(2048, 11008, 4096) == 0      # 688 tiles fill the machine
