@@ -22,16 +22,19 @@
 
 namespace lowbit {
 
-constexpr int RN = 256;        // weight rows per workgroup: 16 tiles
+constexpr int RING_WAVES = 8;  // waves per workgroup; each owns 32 * RNB weight rows (RNB = 1 or 2)
 
 template <int QT> constexpr int ring_hdr_bytes() { return Fmt<QT>::TILE_BYTES - Fmt<QT>::TILE_CODE_BYTES; }
-// one stage: the x block in operand order [16-column step (8)][32-row block (MB)][lane (64)] x 16 B, the
-// code part of the workgroup's 16 tiles, then their header parts
-template <int QT> constexpr int ring_stage_bytes(int mb) { return mb * 8 * 1024 + 16 * Fmt<QT>::TILE_BYTES; }
-// number of stages: 3, or 2 where 3 do not fit 160 KB of LDS.  A deeper ring measured no faster: the
-// loads that a CU can keep in flight are bounded elsewhere.
+// one stage: the x block as 8 * MB pieces of 1 KiB (see the kernel), the code part of the workgroup's
+// 16 tiles, then their header parts
+template <int QT> constexpr int ring_stage_bytes(int mb, int rnb) { return mb * 8 * 1024 + 16 * rnb * Fmt<QT>::TILE_BYTES; }
+// 32 weight rows per wave (256 per workgroup).  64 rows per wave would let an x operand read from LDS
+// feed two MFMAs, but measured 15-60 % slower at every M (sym_int4: [65536 x 4096] at M = 32 / 64 / 128
+// 49 / 62 / 109 us against 42 / 54 / 85), with register spills at 128 rows of x.
+template <int QT> constexpr int ring_rnb(int mb) { return 1; }
+// number of stages: 3, or 2 where 3 do not fit.  A deeper ring measured no faster.
 template <int QT> constexpr int ring_stages(int mb) {
-    const int fit = (160 * 1024 - 64) / ring_stage_bytes<QT>(mb);
+    const int fit = (160 * 1024 - 64) / ring_stage_bytes<QT>(mb, ring_rnb<QT>(mb));
     return fit > 3 ? 3 : fit;
 }
 
@@ -51,21 +54,20 @@ template <int N> __device__ inline void wait_vm() {
 __host__ __device__ inline int64_t ring_first_unit(int64_t b, int64_t U, int64_t B) { return b * U / B; }
 __host__ __device__ inline int64_t ring_owner(int64_t u, int64_t U, int64_t B) { return ((u + 1) * B - 1) / U; }
 
-// RNB = 32-row weight blocks per wave: 2 -> 4 waves of 64 rows, 1 -> 8 waves of 32 rows (two waves
-// per SIMD cover each other's LDS and barrier waits; x is then read from LDS by twice as many waves)
+// MB = 32-row blocks of x per workgroup, RNB = 32-row weight blocks per wave, S = ring stages
 template <int QT, typename AT, int MB, int RNB, int S>
-__global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+__global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                                   AT *__restrict__ y, int M, int N, int K, int seg_slots,
                                                                   float *__restrict__ ws) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
-    constexpr int WAVES = 8 / RNB;
+    constexpr int WAVES = RING_WAVES, NT = 2 * RNB * WAVES, RN = 16 * NT;   // tiles and weight rows per workgroup
     constexpr int XB = MB * 8 * 1024, CODE = F::TILE_CODE_BYTES, HDR = ring_hdr_bytes<QT>();
-    constexpr int STAGE = ring_stage_bytes<QT>(MB);
+    constexpr int STAGE = ring_stage_bytes<QT>(MB, RNB);
     constexpr int CPT = CODE / 1024;                 // 1 KiB code loads per tile
     constexpr int TPI = 256 / HDR;                   // tiles whose headers one 256-byte load covers
     static_assert(TPI >= 1 && TPI <= 4, "header load shape");
-    constexpr int TPW = 16 / WAVES;                  // tiles per wave
+    constexpr int TPW = NT / WAVES;                  // tiles per wave
     constexpr int XL = 8 * MB / WAVES;               // loads per stage and wave: x blocks,
     constexpr int CL = TPW * CPT;                    //   code KiBs,
     constexpr int HL = TPW / TPI > 0 ? TPW / TPI : 1;   // header loads (a wave with fewer tiles than a load covers repeats its neighbour's)
@@ -93,33 +95,37 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
     const int first_tile = u0 / G;
 
     // ---- sources of this lane's share of a stage, for the tile being fetched
-    // x: one load fills the 1 KiB operand block (16-column step ks, row block mb): lane 32*kg + i
-    // fetches row 32*mb + i, columns 16*ks + 8*kg .. +7.  Wave v fills ks = v*XL/MB .. (all mb of each).
-    // weights: wave v owns tiles v*TPW .. of the workgroup's 16 (tile rows past N are clamped: they are
+    // x: one load moves 8 rows x 128 bytes (64 columns) - whole cache lines - into one 1 KiB piece of
+    // LDS: lane (c, i) = 8*c + i fetches the 16 bytes at row 8*t + i, byte 16*c of the half row h.
+    // Piece q = h * 4*MB + t; wave v fills pieces v*XL .. .  The 16 bytes that lane (kg, r) of the MFMA
+    // wants for 16-column step ks and row r of the tile sit in piece (ks/4) * 4*MB + r/8 at
+    // ((ks%4 * 2 + kg) * 8 + r%8) * 16: eight consecutive lanes read 128 contiguous bytes.
+    // weights: wave v owns tiles v*TPW .. of the workgroup's NT (tile rows past N are clamped: they are
     // computed and never stored).  Codes: lane l fetches bytes 16l .. of the tile (and of its second
     // KiB for 8-bit codes).  Headers: one 4-byte load per lane, 256 bytes per instruction, which is
     // the header part of TPI tiles.
-    gbytes xsrc[MB], csrc[TPW], hsrc[HL];
-    constexpr int HFIRST_NUM = 16 / TPI;             // header loads per stage and workgroup
+    gbytes xsrc[XL], csrc[TPW], hsrc[HL];
+    constexpr int HFIRST_NUM = NT / TPI;             // header loads per stage and workgroup
     const int hfirst = wave * HFIRST_NUM / WAVES;    // index of this wave's first header load
     auto set_tile = [&](int tile) {
         const int tile_m = tile % tiles_m, tile_n = tile / tiles_m;
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) {
-            int row = tile_m * 32 * MB + mb * 32 + i32;
+        for (int j = 0; j < XL; j++) {
+            const int q = wave * XL + j, h = q / (4 * MB), t = q % (4 * MB);
+            int row = tile_m * 32 * MB + t * 8 + (lane & 7);
             row = row < M ? row : M - 1;
-            xsrc[mb] = (gbytes)x + ((int64_t)row * K + kg * 8) * (int64_t)sizeof(AT);
+            xsrc[j] = (gbytes)x + ((int64_t)row * K + h * 64 + (lane >> 3) * 8) * (int64_t)sizeof(AT);
         }
 #pragma unroll
         for (int i = 0; i < TPW; i++) {
-            int trow = tile_n * 16 + wave * TPW + i;
+            int trow = tile_n * NT + wave * TPW + i;
             trow = trow < n_tiles ? trow : n_tiles - 1;
             csrc[i] = (gbytes)w + (int64_t)trow * G * F::TILE_BYTES + lane * 16;
         }
 #pragma unroll
         for (int i = 0; i < HL; i++) {
             constexpr int LPT = 64 / TPI;            // lanes per tile
-            int trow = tile_n * 16 + (hfirst + i) * TPI + lane / LPT;
+            int trow = tile_n * NT + (hfirst + i) * TPI + lane / LPT;
             trow = trow < n_tiles ? trow : n_tiles - 1;
             hsrc[i] = (gbytes)w + (int64_t)trow * G * F::TILE_BYTES + CODE + (lane % LPT) * 4;
         }
@@ -134,22 +140,32 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
     auto dma4 = [&](gbytes src, uint32_t lds) {
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
     };
-    auto issue = [&](int kt, int slot) {             // exactly L loads
+    // load j of the L loads of a stage (x blocks first, then code KiBs, then headers); `first` .. `last`
+    // selects a part of them, so that the loads of a stage can be spread over a step
+    auto issue_part = [&](int kt, int slot, const int FIRST, const int LAST) {   // constants once unrolled
         const uint32_t base = __builtin_amdgcn_readfirstlane(ring_base + slot * STAGE);
         const int64_t xk = (int64_t)kt * TILE_COLS * sizeof(AT), wk = (int64_t)kt * F::TILE_BYTES;
 #pragma unroll
         for (int j = 0; j < XL; j++) {
-            const int blk = wave * XL + j;           // (ks, mb) = (blk / MB, blk % MB)
-            dma16(xsrc[j % MB] + xk + (blk / MB) * 16 * sizeof(AT), base + blk * 1024);
+            if (j < FIRST || j >= LAST) continue;
+            dma16(xsrc[j] + xk, base + (wave * XL + j) * 1024);
         }
 #pragma unroll
         for (int i = 0; i < TPW; i++)
 #pragma unroll
-            for (int c = 0; c < CPT; c++) dma16(csrc[i] + wk + c * 1024, base + XB + (wave * TPW + i) * CODE + c * 1024);
+            for (int c = 0; c < CPT; c++) {
+                if (XL + i * CPT + c < FIRST || XL + i * CPT + c >= LAST) continue;
+                dma16(csrc[i] + wk + c * 1024, base + XB + (wave * TPW + i) * CODE + c * 1024);
+            }
 #pragma unroll
-        for (int i = 0; i < HL; i++) dma4(hsrc[i] + wk, base + XB + 16 * CODE + (hfirst + i) * 256);
+        for (int i = 0; i < HL; i++) {
+            if (XL + CL + i < FIRST || XL + CL + i >= LAST) continue;
+            dma4(hsrc[i] + wk, base + XB + NT * CODE + (hfirst + i) * 256);
+        }
     };
-    static_assert(XL % MB == 0 || MB % XL == 0, "x blocks per wave");
+    auto issue = [&](int kt, int slot) {             // exactly L loads
+        issue_part(kt, slot, 0, L);
+    };
 
     struct WRegs {
         TileRegs<QT> lo[RNB], hi[RNB];
@@ -161,7 +177,7 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
         for (int nb = 0; nb < RNB; nb++) {
             const int ti = wave * TPW + nb * 2 + (i32 >> 4);
             const uint8_t *codes = st + ti * CODE;
-            const uint8_t *hdr = st + 16 * CODE + ti * HDR;
+            const uint8_t *hdr = st + NT * CODE + ti * HDR;
             t.lo[nb].q0 = *(const u32x4 *)(codes + slot_lo * 16);
             t.hi[nb].q0 = *(const u32x4 *)(codes + slot_hi * 16);
             if constexpr (F::BITS == 8) {
@@ -217,14 +233,17 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
             asm volatile("s_nop 7\n\ts_nop 4" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[1][0]), "+a"(acc[1][1]),
                          "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[3][0]), "+a"(acc[3][1]));
     };
-    auto compute = [&](const uint8_t *cur, const WRegs &t) {
+    // where the x operand of (16-column step ks, row block mb) starts, and this lane's place in it
+    auto x_piece = [](int ks, int mb) { return ((ks / 4) * 4 * MB + 4 * mb) * 1024 + (ks % 4) * 256; };
+    const int xlane = (i32 >> 3) * 1024 + kg * 128 + (i32 & 7) * 16;
+    auto compute = [&](const uint8_t *cur, const WRegs &t, bool fetch, int f_slot, int f_kt_now) {
         constexpr int PER = 4 / MB;                  // dequantized pairs per MFMA slot
         V8 xv[2][MB];                                // x operands of this 16-column step and the next
         u32x4 wv[RNB];
 #pragma unroll
         for (int k = 0; k < 2; k++)
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) xv[k][mb] = *(const V8 *)(cur + (k * MB + mb) * 1024 + lane * 16);
+            for (int mb = 0; mb < MB; mb++) xv[k][mb] = *(const V8 *)(cur + xlane + x_piece(k, mb));
 #pragma unroll
         for (int nb = 0; nb < RNB; nb++)
 #pragma unroll
@@ -246,13 +265,20 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
                     }
                 }
                 // two steps ahead: one MFMA slot is shorter than the LDS latency when MB is small
-                if (ks < 6) xv[ks & 1][mb] = *(const V8 *)(cur + ((ks + 2) * MB + mb) * 1024 + lane * 16);
+                if (ks < 6) xv[ks & 1][mb] = *(const V8 *)(cur + xlane + x_piece(ks + 2, mb));
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (ks < 7) {
 #pragma unroll
                 for (int nb = 0; nb < RNB; nb++) wv[nb] = wn[nb];
             }
+            // The loads of the stage S - 1 steps ahead go out a few at a time between the 16-column
+            // steps: issued in one burst after the barrier, the eight waves queue up at the address
+            // unit and stand still for about a third of the step.
+            if (fetch) {
+                if ((ks * L) / 8 != ((ks + 1) * L) / 8) issue_part(f_kt_now, f_slot, (ks * L) / 8, ((ks + 1) * L) / 8);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
         acc_guard();
     };
@@ -315,6 +341,13 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
     };
     int f_tile = first_tile, f_kt = u0 - first_tile * G;      // fetch position
     set_tile(f_tile);
+    auto fetched = [&]() {                           // the fetch position moves on by one unit
+        if (++f_kt == G) {
+            f_kt = 0;
+            f_tile++;
+            set_tile(f_tile);                        // one tile past the end at worst: clamped, never fetched
+        }
+    };
     auto issue_next = [&](int slot) {
         issue(f_kt, slot);
         if (++f_kt == G) {
@@ -344,9 +377,10 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (i + S - 1 < n_units) issue_next(fill);
+            const bool fetch = i + S - 1 < n_units;
             read_w(slot, wr);
-            compute(ring + slot * STAGE, wr);
+            compute(ring + slot * STAGE, wr, fetch, fill, f_kt);
+            if (fetch) fetched();
             slot = slot + 1 == S ? 0 : slot + 1;
             fill = fill + 1 == S ? 0 : fill + 1;
         }
@@ -361,7 +395,7 @@ __global__ __launch_bounds__(512 / RNB, 1) void gemm_ring_kernel(const AT *__res
 template <typename AT, int MB, int RNB>
 __global__ __launch_bounds__(256) void ring_reduce_kernel(const float *__restrict__ ws, AT *__restrict__ y, int M, int N,
                                                           int G, int tiles, int B, int seg_slots) {
-    constexpr int WAVES = 8 / RNB, GRP = MB * RNB * 4;
+    constexpr int WAVES = RING_WAVES, GRP = MB * RNB * 4, RN = 32 * RNB * WAVES;
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;       // (tile, wave, group, lane)
     if (t >= (int64_t)tiles * WAVES * GRP * 64) return;
     const int lane = (int)(t & 63);
@@ -390,17 +424,29 @@ __global__ __launch_bounds__(256) void ring_reduce_kernel(const float *__restric
 }
 
 struct RingPlan {
-    int mb, tiles, B, seg_slots;
+    int mb, rnb, tiles, B, seg_slots;
     size_t ws_bytes;
 };
+
+static int ring_rnb_of(int qtype, int mb) {
+    switch (qtype) {
+    case QT_SYM_INT4: return ring_rnb<QT_SYM_INT4>(mb);
+    case QT_ASYM_INT4: return ring_rnb<QT_ASYM_INT4>(mb);
+    case QT_SYM_INT8: return ring_rnb<QT_SYM_INT8>(mb);
+    case QT_NF4: return ring_rnb<QT_NF4>(mb);
+    default: return ring_rnb<QT_FP8_E4M3>(mb);
+    }
+}
 
 // wgs = number of workgroups to deal the units to; 0 = one per CU, but at least four units each (the
 // fixed cost of a workgroup and its partial tile are not worth less).  Without a workspace every
 // workgroup takes whole tiles.
-static RingPlan ring_plan(int M, int N, int K, int wgs, bool have_ws) {
+static RingPlan ring_plan(int M, int N, int K, int rnb, int wgs, bool have_ws) {
     RingPlan p;
     p.mb = M <= 32 ? 1 : M <= 64 ? 2 : 4;
-    p.tiles = ((M + 32 * p.mb - 1) / (32 * p.mb)) * ((N + RN - 1) / RN);
+    p.rnb = rnb;
+    const int rn = 32 * rnb * RING_WAVES;
+    p.tiles = ((M + 32 * p.mb - 1) / (32 * p.mb)) * ((N + rn - 1) / rn);
     const int G = K / TILE_COLS;
     const int64_t U = (int64_t)p.tiles * G;
     int64_t B = wgs > 0 ? wgs : (U / 4 < 256 ? U / 4 : 256);
@@ -411,7 +457,7 @@ static RingPlan ring_plan(int M, int N, int K, int wgs, bool have_ws) {
     // a run of ceil(U/B) units touches at most this many tiles
     const int64_t run = (U + B - 1) / B;
     p.seg_slots = (int)((run + G - 2) / G) + 1;
-    p.ws_bytes = (U % B == 0 && (U / B) % G == 0) ? 0 : (size_t)B * p.seg_slots * (32 * p.mb) * RN * sizeof(float);
+    p.ws_bytes = (U % B == 0 && (U / B) % G == 0) ? 0 : (size_t)B * p.seg_slots * (32 * p.mb) * rn * sizeof(float);
     return p;
 }
 
@@ -419,33 +465,38 @@ static RingPlan ring_plan(int M, int N, int K, int wgs, bool have_ws) {
 // (launch, first loads, partial tiles and their reduction) plus the steps of the longest run; 8-bit
 // codes measured 10% slower.
 double ring_time_us(int M, int N, int K, int qtype, bool have_ws) {
-    const RingPlan p = ring_plan(M, N, K, 0, have_ws);
+    const int mb = M <= 32 ? 1 : M <= 64 ? 2 : 4;
+    const RingPlan p = ring_plan(M, N, K, ring_rnb_of(qtype, mb), 0, have_ws);
     static const double fixed[3] = {11.3, 13.1, 17.3}, step[3] = {1.12, 1.55, 2.56};
     const int i = p.mb == 1 ? 0 : p.mb == 2 ? 1 : 2;
     const int64_t U = (int64_t)p.tiles * (K / TILE_COLS);
-    const double run = (double)((U + p.B - 1) / p.B);
+    const double run = (double)((U + p.B - 1) / p.B) * p.rnb;          // in steps of 256 weight rows
     const double bytes = (qtype == QT_SYM_INT8 || qtype == QT_FP8_E4M3) ? 1.1 : 1.0;
     const double busy = p.B >= 256 ? 1.0 : 0.8 + 0.2 * p.B / 256.0;     // steps are shorter on a machine that is not full
     return fixed[i] - (p.ws_bytes ? 0.0 : 4.5) + run * step[i] * bytes * busy;
 }
 
-size_t ring_workspace_bytes(int M, int N, int K, int wgs) { return ring_plan(M, N, K, wgs, true).ws_bytes; }
+// enough for either tile width
+size_t ring_workspace_bytes(int M, int N, int K, int wgs) {
+    const size_t a = ring_plan(M, N, K, 1, wgs, true).ws_bytes, b = ring_plan(M, N, K, 2, wgs, true).ws_bytes;
+    return a > b ? a : b;
+}
 
 template <int QT, typename AT, int MB, int RNB>
 static int launch_ring_m(const void *x, const void *w, void *y, int M, int N, int K, float *ws, const RingPlan &p,
                          hipStream_t st) {
     constexpr int S = ring_stages<QT>(MB);
-    constexpr int LDS = S * ring_stage_bytes<QT>(MB) + 64;
+    constexpr int LDS = S * ring_stage_bytes<QT>(MB, RNB) + 64;
     auto kern = gemm_ring_kernel<QT, AT, MB, RNB, S>;
     static bool raised = false;                      // the default limit of dynamic LDS is 64 KB
     if (!raised) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) return -6;
         raised = true;
     }
-    hipLaunchKernelGGL(kern, dim3(p.B), dim3(512 / RNB), LDS, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K,
+    hipLaunchKernelGGL(kern, dim3(p.B), dim3(64 * RING_WAVES), LDS, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K,
                        p.seg_slots, ws);
     if (p.ws_bytes) {
-        const int64_t threads = (int64_t)p.tiles * (32 * MB) * RN / 4;
+        const int64_t threads = (int64_t)p.tiles * (32 * MB) * (32 * RNB * RING_WAVES) / 4;
         hipLaunchKernelGGL((ring_reduce_kernel<AT, MB, RNB>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, ws,
                            (AT *)y, M, N, K / TILE_COLS, p.tiles, p.B, p.seg_slots);
     }
@@ -455,9 +506,9 @@ static int launch_ring_m(const void *x, const void *w, void *y, int M, int N, in
 template <int QT, typename AT>
 static int launch_ring_t(const void *x, const void *w, void *y, int M, int N, int K, float *ws, const RingPlan &p,
                          hipStream_t st) {
-    if (p.mb == 1) return launch_ring_m<QT, AT, 1, 1>(x, w, y, M, N, K, ws, p, st);
-    if (p.mb == 2) return launch_ring_m<QT, AT, 2, 1>(x, w, y, M, N, K, ws, p, st);
-    return launch_ring_m<QT, AT, 4, 1>(x, w, y, M, N, K, ws, p, st);
+    if (p.mb == 1) return launch_ring_m<QT, AT, 1, ring_rnb<QT>(1)>(x, w, y, M, N, K, ws, p, st);
+    if (p.mb == 2) return launch_ring_m<QT, AT, 2, ring_rnb<QT>(2)>(x, w, y, M, N, K, ws, p, st);
+    return launch_ring_m<QT, AT, 4, ring_rnb<QT>(4)>(x, w, y, M, N, K, ws, p, st);
 }
 
 template <int QT>
@@ -473,8 +524,9 @@ static int launch_ring_q(const void *x, const void *w, void *y, int dt, int M, i
 int launch_gemm_ring(const void *x, const void *w, void *y, int qtype, int act_dtype, int M, int N, int K,
                      void *workspace, size_t workspace_bytes, int wgs, hipStream_t st) {
     if (M == 0 || N == 0) return 0;
-    RingPlan p = ring_plan(M, N, K, wgs, workspace != nullptr);
-    if (p.ws_bytes > workspace_bytes) p = ring_plan(M, N, K, wgs, false);
+    const int rnb = ring_rnb_of(qtype, M <= 32 ? 1 : M <= 64 ? 2 : 4);
+    RingPlan p = ring_plan(M, N, K, rnb, wgs, workspace != nullptr);
+    if (p.ws_bytes > workspace_bytes) p = ring_plan(M, N, K, rnb, wgs, false);
     float *ws = (float *)workspace;
     switch (qtype) {
     case QT_SYM_INT4: return launch_ring_q<QT_SYM_INT4>(x, w, y, act_dtype, M, N, K, ws, p, st);
