@@ -197,7 +197,8 @@ size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     // enough for whichever kernel lowbit_forward_ws may pick for the shape
     const int s = gemm_splits((int)M, (int)N, (int)K, (size_t)-1);
     const size_t gemm = s > 1 ? split_bytes(M, N, s) : 0;
-    const size_t ring = M <= 512 ? ring_workspace_bytes((int)M, (int)N, (int)K, 0) : 0;
+    const bool ring_range = (double)M * (double)N * (double)K < 3.5e10 || ((M + 127) / 128) * ((N + 255) / 256) <= 256;
+    const size_t ring = ring_range ? ring_workspace_bytes((int)M, (int)N, (int)K, 0) : 0;
     return gemm > ring ? gemm : ring;
 }
 
@@ -220,11 +221,13 @@ static int forward_any(const void *x, const void *w, void *y, int qtype, int lay
     const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
     const int splits = workspace ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
     const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits);
-    // The ring kernel (M up to a few hundred rows, y 8-byte aligned) needs the workspace for its partial
-    // tiles; given that, it measured faster than the tiled GEMM, split or not, up to about 7e10 FLOP
-    // (sym_int4 and sym_int8, seven shapes from [1024 x 8192] to [28672 x 8192], M = 24 .. 512), and
-    // its own estimate decides against the GEMV.
-    if (M <= 512 && !(((uintptr_t)y) & 7) && workspace && (double)M * (double)N * (double)K < 3.5e10 &&
+    // The ring kernel (y 8-byte aligned) needs the workspace for its partial tiles; given that, it measured
+    // faster than the tiled GEMM, split or not, up to about 7e10 FLOP (sym_int4 and sym_int8, seven shapes
+    // from [1024 x 8192] to [28672 x 8192], M = 24 .. 512) and beyond that while the GEMM's 128 x 256 tiles
+    // are no more than one per CU ([4096 x 11008] at M = 2048: 187 against 209 us); its own estimate
+    // decides against the GEMV.
+    const int64_t gemm_tiles = ((M + 127) / 128) * ((N + 255) / 256);
+    if (!(((uintptr_t)y) & 7) && workspace && ((double)M * (double)N * (double)K < 3.5e10 || gemm_tiles <= 256) &&
         ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes) {
         if (ring_time_us((int)M, (int)N, (int)K, qtype, true) < t_gemv)
             return lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, 0, stream);
