@@ -115,6 +115,26 @@ def test_ring_full_size_agrees_with_the_decode_kernel():
         assert d <= 2e-3 * y_gemv.float().abs().max().item()
 
 
+def test_ring_vocabulary_sized_weight_agrees_with_the_decode_kernel():
+    # an lm_head: 125 tiles of 256 rows dealt to 256 workgroups, and K = 11008 (86 steps) with a row
+    # count that leaves the last 32-row block of x partly empty
+    qtype = Q4_0
+    ws = torch.empty(96 << 20, dtype=torch.uint8, device="cuda")
+    for m, n, k in ((40, 32000, 4096), (100, 4096, 11008)):
+        w = torch.randn((n, k), device="cuda") * 0.02
+        blob = torch.empty(ggml.lowbit_blob_bytes(qtype, n * k), dtype=torch.uint8, device="cuda")
+        ggml.lowbit_quantize(w.data_ptr(), blob.data_ptr(), qtype, n, k, TILED, stream())
+        x = (torch.randn((m, k), device="cuda")).bfloat16()
+        y_ring = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        y_gemv = torch.empty_like(y_ring)
+        ggml.lowbit_gemm_ring(x.data_ptr(), blob.data_ptr(), y_ring.data_ptr(), qtype, TILED, 1, m, n, k, ws.data_ptr(),
+                              ws.numel(), 0, stream())
+        ggml.lowbit_gemv(x.data_ptr(), blob.data_ptr(), y_gemv.data_ptr(), qtype, TILED, 1, m, n, k, 0, stream())
+        torch.cuda.synchronize()
+        d = (y_ring.float() - y_gemv.float()).abs().max().item()
+        assert d <= 8e-3 * y_gemv.float().abs().max().item()
+
+
 def test_ring_rejects_bad_arguments():
     m, n, k, qtype = 32, 256, 256, Q4_0
     w = weights(7400, (n, k))
