@@ -232,8 +232,8 @@ def forward_new(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int, 
     y = torch.empty((m, output_size), dtype=xc.dtype, device=x.device)
     if m and output_size:
         with torch.cuda.device(x.device):
-            # split-K workspace for shapes whose output tiles alone do not fill the GPU; taken from
-            # torch's caching allocator, so steady-state calls do not allocate
+            # workspace for the fp32 partial tiles of the batch-size kernel and of the GEMM when it
+            # splits K; taken from torch's caching allocator, so steady-state calls do not allocate
             ws_bytes = ggml.lowbit_workspace_bytes(m, output_size, k) if layout == ggml.LAYOUT_TILED else 0
             ws_bytes = min(ws_bytes, _WORKSPACE_CAP)
             if ws_bytes:
