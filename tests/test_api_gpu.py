@@ -219,11 +219,12 @@ def test_lowbit_linears_replay_correctly_from_a_hip_graph():
     torch.manual_seed(9)
     lins = [_layer(weights(7200 + i, (n, k)), Q["sym_int4"]).to("cuda") for i, (n, k) in
             enumerate([(512, 256), (256, 512)])]
-    emb_like = _layer(weights(7210, (4096, 256)), Q["sym_int8"]).to("cuda")      # many tiles, long K walk
+    emb_like = _layer(weights(7210, (4096, 256)), Q["sym_int8"]).to("cuda")      # many tiles, short K walk
+    tail = _layer(weights(7220, (1024, 4096)), Q["nf4"]).to("cuda")              # few tiles, long K walk: cut tiles
 
     def net(x):
-        return emb_like(lins[1](torch.nn.functional.silu(lins[0](x))))
-    for rows in (1, 48):                                   # GEMV path / split-K GEMM path with a workspace
+        return tail(emb_like(lins[1](torch.nn.functional.silu(lins[0](x)))))
+    for rows in (1, 48):                                   # GEMV path / batch-size kernel with partial tiles in a workspace
         static_x = torch.zeros(rows, 256, dtype=torch.float16, device="cuda")
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
