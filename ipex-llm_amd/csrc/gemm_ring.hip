@@ -391,30 +391,41 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
 }
 
 // Sums the partial tiles of every output tile that was cut into segments and writes y, rounded once.
-// One thread per group of 4 consecutive n, in the order the partial sums were stored.
+// Grid (tiles, pieces of 256 threads): the tile, and with it the list of workgroups that hold a part of
+// it, is the same for a whole workgroup (scalar arithmetic).  One thread per group of 4 consecutive n,
+// in the order the partial sums were stored.
 template <typename AT, int MB, int RNB>
 __global__ __launch_bounds__(256) void ring_reduce_kernel(const float *__restrict__ ws, AT *__restrict__ y, int M, int N,
                                                           int G, int tiles, int B, int seg_slots) {
     constexpr int WAVES = RING_WAVES, GRP = MB * RNB * 4, RN = 32 * RNB * WAVES;
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;       // (tile, wave, group, lane)
-    if (t >= (int64_t)tiles * WAVES * GRP * 64) return;
-    const int lane = (int)(t & 63);
-    const int grp = (int)((t >> 6) % GRP);
-    const int wave = (int)((t >> 6) / GRP % WAVES);
-    const int tile = (int)((t >> 6) / GRP / WAVES);
+    const int tile = blockIdx.x;
+    const int64_t U = (int64_t)tiles * G;
+    const int b0 = (int)ring_owner((int64_t)tile * G, U, B), b1 = (int)ring_owner((int64_t)(tile + 1) * G - 1, U, B);
+    if (b0 == b1) return;                            // one segment covered all of K and wrote y itself
+    const int t = blockIdx.y * 256 + threadIdx.x;    // (wave, group, lane)
+    const int lane = t & 63;
+    const int grp = (t >> 6) % GRP;
+    const int wave = (t >> 6) / GRP;
     const int tiles_m = (M + 32 * MB - 1) / (32 * MB);
     const int mb = grp / (RNB * 4), nb = grp / 4 % RNB, q = grp % 4;
     const int m = (tile % tiles_m) * 32 * MB + mb * 32 + (lane & 31);
     const int n = (tile / tiles_m) * RN + wave * (32 * RNB) + nb * 32 + q * 8 + (lane >> 5) * 4;
     if (m >= M || n >= N) return;
-    const int64_t U = (int64_t)tiles * G;
-    const int b0 = (int)ring_owner((int64_t)tile * G, U, B), b1 = (int)ring_owner((int64_t)(tile + 1) * G - 1, U, B);
-    if (b0 == b1) return;                            // one segment covered all of K and wrote y itself
+    // eight parts in flight at a time (a thread that waited for each part in turn would spend a memory
+    // latency per part); they are added in workgroup order whatever their number
     f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int b = b0; b <= b1; b++) {
-        const int seg = tile - (int)(ring_first_unit(b, U, B) / G);
-        const float *part = ws + ((int64_t)b * seg_slots + seg) * (32 * MB * RN);
-        a += *(const f32x4 *)(part + ((wave * GRP + grp) * 64 + lane) * 4);
+    for (int c = b0; c <= b1; c += 8) {
+        f32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int b = c + j <= b1 ? c + j : b1;
+            const int seg = tile - (int)(ring_first_unit(b, U, B) / G);
+            const float *part = ws + ((int64_t)b * seg_slots + seg) * (32 * MB * RN);
+            v[j] = *(const f32x4 *)(part + (int64_t)t * 4);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (c + j <= b1) a += v[j];
     }
     typedef AT at4 __attribute__((ext_vector_type(4)));
     at4 o;
@@ -496,9 +507,9 @@ static int launch_ring_m(const void *x, const void *w, void *y, int M, int N, in
     hipLaunchKernelGGL(kern, dim3(p.B), dim3(64 * RING_WAVES), LDS, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K,
                        p.seg_slots, ws);
     if (p.ws_bytes) {
-        const int64_t threads = (int64_t)p.tiles * (32 * MB) * (32 * RNB * RING_WAVES) / 4;
-        hipLaunchKernelGGL((ring_reduce_kernel<AT, MB, RNB>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, ws,
-                           (AT *)y, M, N, K / TILE_COLS, p.tiles, p.B, p.seg_slots);
+        constexpr int per_tile = (32 * MB) * (32 * RNB * RING_WAVES) / 4;     // threads: a multiple of 256
+        hipLaunchKernelGGL((ring_reduce_kernel<AT, MB, RNB>), dim3(p.tiles, per_tile / 256), dim3(256), 0, st, ws, (AT *)y,
+                           M, N, K / TILE_COLS, p.tiles, p.B, p.seg_slots);
     }
     return 0;
 }
