@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
                                                         float *__restrict__ ws) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
-    // x block in operand order: [16-column step ks (8)][32-row block (MB32)][lane (64)] x 16 bytes
+    // x block of a K step: 8 * MB32 pieces of 1 KiB (layout below), double buffered
     __shared__ __attribute__((aligned(16))) uint8_t xs0[8 * MB32 * 1024];
     __shared__ __attribute__((aligned(16))) uint8_t xs1[8 * MB32 * 1024];
     __shared__ float lut[16];
@@ -102,13 +102,23 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         wt[nb] = (gbytes)w + (int64_t)trow * G * F::TILE_BYTES;
     }
 
-    // x goes global -> registers -> LDS.  Per K step the workgroup copies 128 rows x 256 bytes;
-    // a wave-wide load covers 16 rows x 64 bytes: chunk = 4*wave + lane/16 (16 bytes each), row =
-    // 16*i + lane%16 for i = 0..7.  The chunk lands where the B operand wants it:
-    // step ks = chunk/2, kg = chunk%2, block row/32, lane slot 32*kg + row%32.
+    // The x block of a K step (128 rows x 256 bytes) sits in LDS as 32 pieces of 1 KiB: piece h * 16 + t
+    // holds rows 8t .. 8t+7 of the half row h (64 columns = 128 bytes), the 16 bytes of (row r, 16-byte
+    // chunk c) at (c * 8 + r % 8) * 16.  Lane (kg, i) of the MFMA reads, for 16-column step ks and row
+    // block mb, piece (ks/4) * 16 + 4*mb + i/8 at ((ks%4 * 2 + kg) * 8 + i%8) * 16: eight consecutive
+    // lanes read 128 contiguous bytes.  The layout is chosen for the DMA form below.
+    //
+    // Register-staged form: x goes global -> registers -> LDS; a wave-wide load covers 16 rows x 64
+    // bytes: chunk = 4*wave + lane/16 (16 bytes each), row = 16*i + lane%16 for i = 0..7.
     const int chunk = wave * 4 + (lane >> 4);
-    uint32_t xoff[DMA ? MB32 : 8];
+    uint32_t xoff[DMA ? 1 : 8];
     int xl[DMA ? 1 : 8];
+    // DMA form: x goes global -> LDS without passing through registers.  One wave-wide instruction
+    // fills one piece: lane 8*c + i fetches the 16 bytes at row 8t + i, byte 16c of the half row - whole
+    // 128-byte lines, 8 per instruction - and the hardware writes the lanes to LDS in lane order.  Wave
+    // w fills pieces 8w .. 8w+7: half row w/2, rows 64*(w%2) + 8j + i.  Rows past M are clamped (the
+    // offsets are formed with 24-bit multiplies: the launcher keeps M and 2K below 2^24).
+    uint32_t xrow0 = 0, xcol = 0;
     if constexpr (!DMA) {
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -116,19 +126,11 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             int row = m0 + row_in;
             row = row < M ? row : M - 1;
             xoff[i] = (uint32_t)(((int64_t)row * K + chunk * 8) * (int64_t)sizeof(AT));
-            xl[i] = (((chunk >> 1) * MB32 + (row_in >> 5)) * 64 + (chunk & 1) * 32 + (row_in & 31)) * 16;
+            xl[i] = (((chunk >> 3) * (4 * MB32) + (row_in >> 3)) * 64 + (chunk & 7) * 8 + (row_in & 7)) * 16;
         }
     } else {
-        // DMA form: x goes global -> LDS without passing through registers.  One wave-wide
-        // instruction fills one 1 KiB operand block (16-column step ks, 32-row block mb): lane
-        // 32*kg + i fetches the 16 bytes at row 32*mb + i, columns 16*ks + 8*kg, and the hardware
-        // writes the lanes to LDS in lane order.  Wave w fills blocks 8w .. 8w+7 (ks = 2w, 2w+1).
-#pragma unroll
-        for (int mb = 0; mb < MB32; mb++) {
-            int row = m0 + mb * 32 + i32;
-            row = row < M ? row : M - 1;
-            xoff[mb] = (uint32_t)(((int64_t)row * K + kg * 8) * (int64_t)sizeof(AT));
-        }
+        xrow0 = m0 + 64 * (wave & 1) + (lane & 7);
+        xcol = (wave >> 1) * 128 + (lane >> 3) * 16;
     }
     // Split-K: with a workspace the grid has a second dimension, workgroup (t, s) walks the K steps
     // s * k_steps .. and leaves its fp32 partial tile in ws[s]; a second kernel sums the splits.  It
@@ -136,20 +138,26 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
     const int kt0 = ws ? blockIdx.y * k_steps : 0;
     const int Gs = ws ? (k_steps < G - kt0 ? k_steps : G - kt0) : G;
     const int last = Gs - 1;
-    auto dma_x = [&](int kt, uint8_t *buf) {
+    // the same loads one at a time, for spreading them over a step: a burst of 8 + 6 loads per wave,
+    // from eight waves at once, queues up at the CU's address unit and the waves stand still meanwhile
+    // (measured with cycle counters: 41 % of a K step at M = 2048)
+    auto dma_x_one = [&](int kt, uint8_t *buf, int j) {
         kt = kt0 + (kt < last ? kt : last);
-        const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT) + wave * 2 * 16 * sizeof(AT);
         // Issued from inline assembly: the compiler's wait-count pass treats an LDS-DMA as aliasing
         // every later LDS access and would wait for it immediately.  Completion is awaited by the
         // explicit vmcnt(0) ahead of the workgroup barrier that publishes the buffer.
+        const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
         const uint32_t lbase = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + wave * 8 * 1024);
+        uint32_t row = xrow0 + 8 * j;
+        row = row < (uint32_t)M ? row : (uint32_t)M - 1;
+        const uint8_t *src = xk + (__umul24(row, (uint32_t)K * (uint32_t)sizeof(AT)) + xcol);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :: "v"(src), "s"(lbase + j * 1024) : "memory", "m0");
+    };
+    auto dma_x = [&](int kt, uint8_t *buf) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const uint8_t *src = xk + xoff[DMA ? (j & 3) : 0] + (j >> 2) * 16 * sizeof(AT);
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                         :: "v"(src), "s"(lbase + j * 1024) : "memory", "m0");
-        }
+        for (int j = 0; j < 8; j++) dma_x_one(kt, buf, j);
     };
     auto load_x = [&](int kt, u32x4 (&xr)[8]) {
         kt = kt0 + (kt < last ? kt : last);              // past the end: a harmless re-read, never used
@@ -173,6 +181,14 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             t.hi[nb].q0 = ld<u32x4>(tile + slot_hi * 16);
             if constexpr (F::BITS == 8) t.hi[nb].q1 = ld<u32x4>(tile + 1024 + slot_hi * 16);
         }
+    };
+
+    auto load_w_nb = [&](int kt, WRegs &t, int nb) {
+        kt = kt0 + (kt < last ? kt : last);
+        const gbytes tile = wt[nb] + (int64_t)kt * F::TILE_BYTES;
+        load_tile<QT>(tile, slot_lo, r16, t.lo[nb]);
+        t.hi[nb].q0 = ld<u32x4>(tile + slot_hi * 16);
+        if constexpr (F::BITS == 8) t.hi[nb].q1 = ld<u32x4>(tile + 1024 + slot_hi * 16);
     };
 
     f32x16 acc[MB32][NB32];
@@ -199,13 +215,15 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
     // the next step's weights are dequantized after every MFMA, so that LDS latency and the VALU
     // work run in the shadow of the MFMA pipe.  MBC = number of 32-row blocks of x that take part
     // (a compile-time constant: a branch around each MFMA would cut the schedule into pieces).
-    auto compute = [&](const uint8_t *cur, const WRegs &t, auto mbc_) {
+    auto x_piece = [](int ks, int mb) { return ((ks / 4) * 4 * MB32 + 4 * mb) * 1024 + (ks % 4) * 256; };
+    const int xlane = (i32 >> 3) * 1024 + kg * 128 + (i32 & 7) * 16;
+    auto compute = [&](const uint8_t *cur, const WRegs &t, auto mbc_, auto &&between) {
         constexpr int MBC = decltype(mbc_)::value;
         constexpr int PER = (4 * NB32) / (MBC * NB32);        // dequantized pairs per MFMA slot
         V8 xv[MBC];
         u32x4 wv[NB32];
 #pragma unroll
-        for (int mb = 0; mb < MBC; mb++) xv[mb] = *(const V8 *)(cur + mb * 1024 + lane * 16);
+        for (int mb = 0; mb < MBC; mb++) xv[mb] = *(const V8 *)(cur + xlane + x_piece(0, mb));
 #pragma unroll
         for (int nb = 0; nb < NB32; nb++)
 #pragma unroll
@@ -226,11 +244,13 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
                         }
                     }
                 }
-                if (ks < 7) xv[mb] = *(const V8 *)(cur + ((ks + 1) * MB32 + mb) * 1024 + lane * 16);
+                if (ks < 7) xv[mb] = *(const V8 *)(cur + xlane + x_piece(ks + 1, mb));
                 // keep this order: the scheduler does not know how long an MFMA takes and would
                 // sink the LDS read down to its first use, exposing the LDS latency every time
                 __builtin_amdgcn_sched_barrier(0);
             }
+            between(ks);
+            __builtin_amdgcn_sched_barrier(0);
             if (ks < 7) {
 #pragma unroll
                 for (int nb = 0; nb < NB32; nb++) wv[nb] = wn[nb];
@@ -238,6 +258,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         }
     };
     typedef std::integral_constant<int, MB32> full_t;
+    auto nothing = [](int) {};
 
     auto epilogue = [&](auto mbc_) {
         constexpr int MBC = decltype(mbc_)::value;
@@ -300,18 +321,22 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             wait_all_loads();
             __syncthreads();
             for (int kt = 0; kt + 1 < Gs; kt += 2) {
-                dma_x(kt + 1, xs1);
-                load_w(kt + 1, w1);
-                compute(xs0, w0, mbc);
+                compute(xs0, w0, mbc, [&](int ks) {
+                    dma_x_one(kt + 1, xs1, ks);
+                    if (ks == 2) load_w_nb(kt + 1, w1, 0);
+                    if (ks == 5) load_w_nb(kt + 1, w1, 1);
+                });
                 wait_all_loads();
                 __syncthreads();
-                dma_x(kt + 2, xs0);                          // past the end: a clamped, unused re-read
-                load_w(kt + 2, w0);
-                compute(xs1, w1, mbc);
+                compute(xs1, w1, mbc, [&](int ks) {          // past the end: clamped, unused re-reads
+                    dma_x_one(kt + 2, xs0, ks);
+                    if (ks == 2) load_w_nb(kt + 2, w0, 0);
+                    if (ks == 5) load_w_nb(kt + 2, w0, 1);
+                });
                 wait_all_loads();
                 __syncthreads();
             }
-            if (Gs & 1) compute(xs0, w0, mbc);
+            if (Gs & 1) compute(xs0, w0, mbc, nothing);
         };
         // tail tiles and small expert groups: 32-row blocks without rows of x skip their MFMAs
         const int mb_cnt = (M - m0 + 31) / 32;
@@ -343,7 +368,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
     if (kt + (i) < Gs) {                                \
         load_x(kt + (i) + 2, xld);                      \
         load_w(kt + (i) + 2, wl);                       \
-        compute(cur, wc, full_t());                     \
+        compute(cur, wc, full_t(), nothing);            \
         store_x(nxt, xst);                              \
         __syncthreads();                                \
     }
@@ -446,7 +471,7 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     // vector registers) lets a CU hold two workgroups that cover each other's waits; it wins as
     // soon as there are more workgroups than CUs.  With at most one per CU the register-staged
     // form with its deeper prefetch is faster.
-    const bool dma = tiles_m * tiles_n * ny > 256;
+    const bool dma = tiles_m * tiles_n * ny > 256 && M < (1 << 24) && K < (1 << 23);   // 24-bit row offsets
     if (dma)
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
                            (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0,
@@ -486,6 +511,7 @@ static int launch_grouped_q(const void *x, const void *const *w, void *y, const 
 int launch_grouped_gemm(const void *x, const void *const *w, void *y, const int32_t *offsets, int n_groups,
                         int total_rows, int qtype, int act_dtype, int N, int K, hipStream_t st) {
     if (total_rows == 0 || N == 0 || n_groups == 0) return 0;
+    if (total_rows >= (1 << 24) || K >= (1 << 23)) return -3;        // 24-bit row offsets in the kernel
     switch (qtype) {
     case QT_SYM_INT4: return launch_grouped_q<QT_SYM_INT4>(x, w, y, offsets, n_groups, total_rows, act_dtype, N, K, st);
     case QT_ASYM_INT4: return launch_grouped_q<QT_ASYM_INT4>(x, w, y, offsets, n_groups, total_rows, act_dtype, N, K, st);
