@@ -191,6 +191,19 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         if constexpr (F::BITS == 8) t.hi[nb].q1 = ld<u32x4>(tile + 1024 + slot_hi * 16);
     };
 
+    // what goes out after 16-column step ks: everything within the first five of the eight steps, so
+    // that the data has the rest of the K step to arrive (later placements end in a longer wait at
+    // the barrier, a single burst at ks = 0 stalls the waves at the address unit)
+    auto fetch_part = [&](int kt, uint8_t *buf, WRegs &t, int ks) {
+        if (ks < 2) {
+            load_w_nb(kt, t, ks);
+            dma_x_one(kt, buf, ks);
+        } else if (ks < 5) {
+            dma_x_one(kt, buf, 2 * ks - 2);
+            dma_x_one(kt, buf, 2 * ks - 1);
+        }
+    };
+
     f32x16 acc[MB32][NB32];
 #pragma unroll
     for (int mb = 0; mb < MB32; mb++)
@@ -322,16 +335,12 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             __syncthreads();
             for (int kt = 0; kt + 1 < Gs; kt += 2) {
                 compute(xs0, w0, mbc, [&](int ks) {
-                    dma_x_one(kt + 1, xs1, ks);
-                    if (ks == 2) load_w_nb(kt + 1, w1, 0);
-                    if (ks == 5) load_w_nb(kt + 1, w1, 1);
+                    fetch_part(kt + 1, xs1, w1, ks);
                 });
                 wait_all_loads();
                 __syncthreads();
                 compute(xs1, w1, mbc, [&](int ks) {          // past the end: clamped, unused re-reads
-                    dma_x_one(kt + 2, xs0, ks);
-                    if (ks == 2) load_w_nb(kt + 2, w0, 0);
-                    if (ks == 5) load_w_nb(kt + 2, w0, 1);
+                    fetch_part(kt + 2, xs0, w0, ks);
                 });
                 wait_all_loads();
                 __syncthreads();
