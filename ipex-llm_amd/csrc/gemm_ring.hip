@@ -51,14 +51,19 @@ template <int N> __device__ inline void wait_vm() {
 // b*U/B .. (b+1)*U/B - 1.  A run may cross from one tile into the next; each piece of a tile
 // ("segment") that does not cover all of K leaves an fp32 partial tile in the workspace, in slot
 // b * seg_slots + (tile - first tile of b).
-__host__ __device__ inline int64_t ring_first_unit(int64_t b, int64_t U, int64_t B) { return b * U / B; }
-__host__ __device__ inline int64_t ring_owner(int64_t u, int64_t U, int64_t B) { return ((u + 1) * B - 1) / U; }
+// With q = U / B and r = U % B the first r workgroups take q + 1 units, the others q: no division on the
+// device beyond 32-bit ones.
+__host__ __device__ inline int ring_first_unit(int b, int q, int r) { return b * q + (b < r ? b : r); }
+__host__ __device__ inline int ring_owner(int u, int q, int r) {
+    const int big = r * (q + 1);                     // units held by the workgroups with q + 1
+    return u < big ? u / (q + 1) : r + (u - big) / q;
+}
 
 // MB = 32-row blocks of x per workgroup, RNB = 32-row weight blocks per wave, S = ring stages
 template <int QT, typename AT, int MB, int RNB, int S>
 __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                                   AT *__restrict__ y, int M, int N, int K, int seg_slots,
-                                                                  float *__restrict__ ws) {
+                                                                  int run_q, int run_r, float *__restrict__ ws) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
     constexpr int WAVES = RING_WAVES, NT = 2 * RNB * WAVES, RN = 16 * NT;   // tiles and weight rows per workgroup
@@ -89,8 +94,7 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
     const int kg = lane >> 5, i32 = lane & 31, r16 = lane & 15;
     const int slot_lo = kg * 16 + r16, slot_hi = (kg + 2) * 16 + r16;
 
-    const int64_t U = (int64_t)tiles_m * tiles_n * G;
-    const int u0 = (int)ring_first_unit(blockIdx.x, U, gridDim.x), u1 = (int)ring_first_unit(blockIdx.x + 1, U, gridDim.x);
+    const int u0 = ring_first_unit(blockIdx.x, run_q, run_r), u1 = ring_first_unit(blockIdx.x + 1, run_q, run_r);
     const int n_units = u1 - u0;
     const int first_tile = u0 / G;
 
@@ -396,11 +400,10 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
 // in the order the partial sums were stored.
 template <typename AT, int MB, int RNB>
 __global__ __launch_bounds__(256) void ring_reduce_kernel(const float *__restrict__ ws, AT *__restrict__ y, int M, int N,
-                                                          int G, int tiles, int B, int seg_slots) {
+                                                          int G, int run_q, int run_r, int seg_slots) {
     constexpr int WAVES = RING_WAVES, GRP = MB * RNB * 4, RN = 32 * RNB * WAVES;
     const int tile = blockIdx.x;
-    const int64_t U = (int64_t)tiles * G;
-    const int b0 = (int)ring_owner((int64_t)tile * G, U, B), b1 = (int)ring_owner((int64_t)(tile + 1) * G - 1, U, B);
+    const int b0 = ring_owner(tile * G, run_q, run_r), b1 = ring_owner((tile + 1) * G - 1, run_q, run_r);
     if (b0 == b1) return;                            // one segment covered all of K and wrote y itself
     const int t = blockIdx.y * 256 + threadIdx.x;    // (wave, group, lane)
     const int lane = t & 63;
@@ -419,7 +422,7 @@ __global__ __launch_bounds__(256) void ring_reduce_kernel(const float *__restric
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const int b = c + j <= b1 ? c + j : b1;
-            const int seg = tile - (int)(ring_first_unit(b, U, B) / G);
+            const int seg = tile - ring_first_unit(b, run_q, run_r) / G;
             const float *part = ws + ((int64_t)b * seg_slots + seg) * (32 * MB * RN);
             v[j] = *(const f32x4 *)(part + (int64_t)t * 4);
         }
@@ -504,12 +507,15 @@ static int launch_ring_m(const void *x, const void *w, void *y, int M, int N, in
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) return -6;
         raised = true;
     }
+    const int64_t U = (int64_t)p.tiles * (K / TILE_COLS);
+    if (U >= (int64_t)1 << 31) return -3;
+    const int run_q = (int)(U / p.B), run_r = (int)(U % p.B);
     hipLaunchKernelGGL(kern, dim3(p.B), dim3(64 * RING_WAVES), LDS, st, (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K,
-                       p.seg_slots, ws);
+                       p.seg_slots, run_q, run_r, ws);
     if (p.ws_bytes) {
         constexpr int per_tile = (32 * MB) * (32 * RNB * RING_WAVES) / 4;     // threads: a multiple of 256
         hipLaunchKernelGGL((ring_reduce_kernel<AT, MB, RNB>), dim3(p.tiles, per_tile / 256), dim3(256), 0, st, ws, (AT *)y,
-                           M, N, K / TILE_COLS, p.tiles, p.B, p.seg_slots);
+                           M, N, K / TILE_COLS, run_q, run_r, p.seg_slots);
     }
     return 0;
 }
