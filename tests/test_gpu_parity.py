@@ -272,6 +272,15 @@ def test_device_entry_points_reject_bad_arguments():
     with pytest.raises(RuntimeError, match="tiled"):           # 24 rows cannot be tiled
         ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 2, 24, 256,
                             stream())
+    # the dequantizers store 16 bytes per lane: a misaligned destination is refused, not mis-stored
+    out = torch.empty(32 * 256 + 8, dtype=torch.float16, device="cuda")
+    rows = torch.zeros(4, dtype=torch.int64, device="cuda")
+    ggml.lowbit_dequantize(blob.data_ptr(), out.data_ptr(), Q4_0, 32, 256, TILED, DT[torch.float16], stream())
+    with pytest.raises(RuntimeError, match="misaligned"):
+        ggml.lowbit_dequantize(blob.data_ptr(), out.data_ptr() + 2, Q4_0, 32, 256, TILED, DT[torch.float16], stream())
+    with pytest.raises(RuntimeError, match="misaligned"):
+        ggml.lowbit_dequantize_rows(blob.data_ptr(), rows.data_ptr(), 4, out.data_ptr() + 8, Q4_0, 32, 256, TILED,
+                                    DT[torch.float16], stream())
     # empty problems are no-ops
     ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 0, 32, 256, stream())
     ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), Q4_0, TILED, DT[torch.float16], 2, 0, 256, stream())
