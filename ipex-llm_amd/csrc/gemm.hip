@@ -165,6 +165,10 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
 #pragma unroll
         for (int i = 0; i < 8; i++) xr[i] = *(const u32x4 *)(xk + xoff[i]);
     };
+    auto load_x_one = [&](int kt, u32x4 (&xr)[8], int i) {
+        kt = kt0 + (kt < last ? kt : last);
+        xr[i] = *(const u32x4 *)((const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT) + xoff[DMA ? 0 : i]);
+    };
     auto store_x = [&](uint8_t *buf, const u32x4 (&xr)[8]) {
 #pragma unroll
         for (int i = 0; i < 8; i++) *(u32x4 *)(buf + xl[i]) = xr[i];
@@ -373,13 +377,14 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
     store_x(xs0, xa);
     __syncthreads();
 
-#define LOWBIT_GEMM_STEP(i, cur, nxt, xst, xld, wc, wl) \
-    if (kt + (i) < Gs) {                                \
-        load_x(kt + (i) + 2, xld);                      \
-        load_w(kt + (i) + 2, wl);                       \
-        compute(cur, wc, full_t(), nothing);            \
-        store_x(nxt, xst);                              \
-        __syncthreads();                                \
+#define LOWBIT_GEMM_STEP(i, cur, nxt, xst, xld, wc, wl)                        \
+    if (kt + (i) < Gs) {                                                       \
+        compute(cur, wc, full_t(), [&](int ks) {                               \
+            if (ks < 2) load_w_nb(kt + (i) + 2, wl, ks);                       \
+            load_x_one(kt + (i) + 2, xld, ks);                                 \
+        });                                                                    \
+        store_x(nxt, xst);                                                     \
+        __syncthreads();                                                       \
     }
     for (int kt = 0; kt < Gs; kt += 6) {
         LOWBIT_GEMM_STEP(0, xs0, xs1, xb, xa, w0, w2)
