@@ -191,14 +191,21 @@ int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout,
                       stream);
 }
 
+// shapes for which lowbit_forward_ws considers the ring kernel (see forward_any)
+static bool ring_range(int qtype, int64_t M, int64_t N, int64_t K) {
+    const bool small = (double)M * (double)N * (double)K < 3.5e10;
+    if (qtype == LOWBIT_QT_NF4) return small || ((M + 127) / 128) * ((N + 255) / 256) <= 256;
+    return small && M < 512;
+}
+
 size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 16 || N <= 0 || K < 128 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;   // M <= 16: GEMV
     if (N % 16 || K % 128) return 0;                                                                  // not tileable: GEMV
     // enough for whichever kernel lowbit_forward_ws may pick for the shape
     const int s = gemm_splits((int)M, (int)N, (int)K, (size_t)-1);
     const size_t gemm = s > 1 ? split_bytes(M, N, s) : 0;
-    const bool ring_range = (double)M * (double)N * (double)K < 3.5e10 || ((M + 127) / 128) * ((N + 255) / 256) <= 256;
-    const size_t ring = ring_range ? ring_workspace_bytes((int)M, (int)N, (int)K, 0) : 0;
+    // the query carries no qtype: the widest range any format uses
+    const size_t ring = ring_range(LOWBIT_QT_NF4, M, N, K) ? ring_workspace_bytes((int)M, (int)N, (int)K, 0) : 0;
     return gemm > ring ? gemm : ring;
 }
 
@@ -222,12 +229,12 @@ static int forward_any(const void *x, const void *w, void *y, int qtype, int lay
     const int splits = workspace ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
     const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits);
     // The ring kernel (y 8-byte aligned) needs the workspace for its partial tiles; given that, it measured
-    // faster than the tiled GEMM, split or not, up to about 7e10 FLOP (sym_int4 and sym_int8, seven shapes
-    // from [1024 x 8192] to [28672 x 8192], M = 24 .. 512) and beyond that while the GEMM's 128 x 256 tiles
-    // are no more than one per CU ([4096 x 11008] at M = 2048: 187 against 209 us); its own estimate
-    // decides against the GEMV.
-    const int64_t gemm_tiles = ((M + 127) / 128) * ((N + 255) / 256);
-    if (!(((uintptr_t)y) & 7) && workspace && ((double)M * (double)N * (double)K < 3.5e10 || gemm_tiles <= 256) &&
+    // faster than or level with the tiled GEMM, split or not, below M = 512 and about 7e10 FLOP (sym_int4 and
+    // sym_int8, seven shapes from [1024 x 8192] to [28672 x 8192]).  With nf4, whose code-book lookups weigh
+    // on the GEMM's tighter loop, it stays ahead at larger M as well while the GEMM's tiles are no more
+    // than one per CU (Llama-3-70B set at M = 512 / 1024: 755 / 808 against 706 / 761 TFLOP/s).  Its own
+    // estimate decides against the GEMV.
+    if (!(((uintptr_t)y) & 7) && workspace && ring_range(qtype, M, N, K) &&
         ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes) {
         if (ring_time_us((int)M, (int)N, (int)K, qtype, true) < t_gemv)
             return lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, 0, stream);
