@@ -502,11 +502,11 @@ static int launch_ring_m(const void *x, const void *w, void *y, int M, int N, in
     constexpr int S = ring_stages<QT>(MB);
     constexpr int LDS = S * ring_stage_bytes<QT>(MB, RNB) + 64;
     auto kern = gemm_ring_kernel<QT, AT, MB, RNB, S>;
-    static bool raised = false;                      // the default limit of dynamic LDS is 64 KB
-    if (!raised) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) return -6;
-        raised = true;
-    }
+    // the default limit of dynamic LDS is 64 KB; raised once per process (thread-safe static), on the one GPU
+    // this library drives
+    static const hipError_t raised =
+        hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    if (raised != hipSuccess) return -6;
     const int64_t U = (int64_t)p.tiles * (K / TILE_COLS);
     if (U >= (int64_t)1 << 31) return -3;
     const int run_q = (int)(U / p.B), run_r = (int)(U % p.B);
