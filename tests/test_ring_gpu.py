@@ -157,3 +157,28 @@ def test_ring_rejects_bad_arguments():
     bad(9, x.data_ptr() + 4, "workspace")
     ggml.lowbit_gemm_ring(*ok)
     torch.cuda.synchronize()
+
+
+def test_forward_ws_random_shapes_against_oracle():
+    # whatever kernel the library picks for 40 seeded random problems (all qtypes, both activation types,
+    # M from 1 to 600, ragged N and K in tile units), with the workspace it asks for
+    rng = np.random.default_rng(77)
+    for case in range(40):
+        qtype = ALL[case % len(ALL)]
+        dtype = (torch.float16, torch.bfloat16)[(case // len(ALL)) % 2]
+        m = int(rng.choice([1, 3, 16, 17, 31, 33, 64, 65, 100, 128, 129, 200, 257, 400, 512, 600]))
+        n = 16 * int(rng.integers(1, 65))
+        k = 128 * int(rng.integers(1, 17))
+        w = weights(9000 + case, (n, k))
+        x = acts(9100 + case, m, k, dtype)
+        blob = dev_quantize(w, qtype, TILED)
+        need = ggml.lowbit_workspace_bytes(m, n, k)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        y = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        ggml.lowbit_forward_ws(x.cuda().data_ptr(), blob.data_ptr(), y.data_ptr(), qtype, TILED, DT[dtype], m, n, k,
+                               ws.data_ptr(), need, stream())
+        torch.cuda.synchronize()
+        y_exact = orc.mul_mat_exact(orc.quantize(w, qtype), x.float().numpy(), (n, k), qtype)
+        got = y.float().cpu().numpy()
+        assert np.isfinite(got).all(), (case, qtype, m, n, k)
+        assert np.abs(got - y_exact).max() <= _tol(dtype) * np.abs(y_exact).max(), (case, qtype, m, n, k)
