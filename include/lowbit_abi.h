@@ -96,6 +96,62 @@ void ggml_compute_forward_mul_mat_q_fp32(const int64_t *src0_ne, const void *src
 /* llama_cpp.py:1189-1193.  Selects device 0 and loads the kernels. */
 void llama_init_backend(void);
 
+/* llama_cpp.py:970-1047: quantizers for k-quants (importance weights) and for the NPU.  Not implemented:
+ * they return 0 bytes written and leave a text for lowbit_last_error(). */
+size_t ggml_quantize_tensor_with_weights(const float *src, void *dst, int qtype, int nrow, int n_per_row, int64_t *hist,
+                                         const float *weights);
+size_t ggml_quantize_tensor_rtn(const float *src, void *dst, float *scale, int qtype, size_t n, int k, int64_t *hist,
+                                bool scale_search);
+size_t ggml_quantize_tensor_rtn_with_weights(const float *src, void *dst, float *scale, int qtype, size_t n, int k,
+                                             int64_t *hist, bool scale_search, const float *weights);
+/* llama_cpp.py:1081 resolves this name (a restype assignment, no prototype, no caller).  Placeholder that aborts. */
+void ggml_quantize_q4_0(void);
+/* llama.cpp's model API, resolved by llama_cpp.py:228-940 at import and outside the low-bit linear path.
+ * Exported so that the import succeeds with LLAMA_CPP_LIB pointing here; the real prototypes differ - these
+ * are placeholders that print the name and abort when called. */
+void llama_apply_lora_from_file(void);
+void llama_context_default_params(void);
+void llama_copy_state_data(void);
+void llama_eval(void);
+void llama_free(void);
+void llama_get_embeddings(void);
+void llama_get_kv_cache_token_count(void);
+void llama_get_logits(void);
+void llama_get_state_size(void);
+void llama_init_candidates(void);
+void llama_init_from_file(void);
+void llama_load_session_file(void);
+void llama_mlock_supported(void);
+void llama_mmap_supported(void);
+void llama_model_quantize(void);
+void llama_n_ctx(void);
+void llama_n_embd(void);
+void llama_n_vocab(void);
+void llama_print_system_info(void);
+void llama_print_timings(void);
+void llama_reset_timings(void);
+void llama_sample_frequency_and_presence_penalties(void);
+void llama_sample_repetition_penalty(void);
+void llama_sample_softmax(void);
+void llama_sample_tail_free(void);
+void llama_sample_temperature(void);
+void llama_sample_token(void);
+void llama_sample_token_greedy(void);
+void llama_sample_token_mirostat(void);
+void llama_sample_token_mirostat_v2(void);
+void llama_sample_top_k(void);
+void llama_sample_top_p(void);
+void llama_sample_typical(void);
+void llama_save_session_file(void);
+void llama_set_rng_seed(void);
+void llama_set_state_data(void);
+void llama_time_us(void);
+void llama_token_bos(void);
+void llama_token_eos(void);
+void llama_token_nl(void);
+void llama_token_to_str(void);
+void llama_tokenize(void);
+
 /* ------------------------------------------------------------------ (2) */
 
 /* Bytes of a blob holding n_weights weights; 0 for an unknown qtype. */

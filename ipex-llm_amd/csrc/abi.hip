@@ -439,4 +439,74 @@ void llama_init_backend(void) {
     (void)check_hip(hipSetDevice(0), "hipSetDevice");
 }
 
+
+// ------------------------------------------------ symbols the reference resolves but this path does not serve
+//
+// python/llm/src/ipex_llm/ggml/model/llama/llama_cpp.py touches every one of these at import
+// (`_lib.<name>.argtypes = ...`), so a library named by LLAMA_CPP_LIB has to export them or the import
+// raises AttributeError.  The quantizers for k-quants and the NPU return 0 bytes written with an error
+// text; llama.cpp's model API (tokenizer, eval, sampling, sessions) is not part of a low-bit linear
+// library: those stubs say so and abort, the reference's convention for failures inside native code.
+size_t ggml_quantize_tensor_with_weights(const float *, void *, int qtype, int, int, int64_t *, const float *) {
+    fail(LOWBIT_EQTYPE, "ggml_quantize_tensor_with_weights: importance-weighted (k-quant) quantizers are not implemented (qtype %d)", qtype);
+    return 0;
+}
+size_t ggml_quantize_tensor_rtn(const float *, void *, float *, int qtype, size_t, int, int64_t *, bool) {
+    fail(LOWBIT_EQTYPE, "ggml_quantize_tensor_rtn: the NPU quantizer is not implemented (qtype %d)", qtype);
+    return 0;
+}
+size_t ggml_quantize_tensor_rtn_with_weights(const float *, void *, float *, int qtype, size_t, int, int64_t *, bool,
+                                             const float *) {
+    fail(LOWBIT_EQTYPE, "ggml_quantize_tensor_rtn_with_weights: the NPU quantizer is not implemented (qtype %d)", qtype);
+    return 0;
+}
+[[noreturn]] static void absent(const char *name) {
+    fprintf(stderr, "liblowbit_hip: %s is not provided by this library (low-bit linear path only)\n", name);
+    abort();
+}
+// llama_cpp.py:1081 sets a restype on it (and nothing else); no caller in the reference
+void ggml_quantize_q4_0(void) { absent("ggml_quantize_q4_0"); }
+void llama_apply_lora_from_file(void) { absent("llama_apply_lora_from_file"); }
+void llama_context_default_params(void) { absent("llama_context_default_params"); }
+void llama_copy_state_data(void) { absent("llama_copy_state_data"); }
+void llama_eval(void) { absent("llama_eval"); }
+void llama_free(void) { absent("llama_free"); }
+void llama_get_embeddings(void) { absent("llama_get_embeddings"); }
+void llama_get_kv_cache_token_count(void) { absent("llama_get_kv_cache_token_count"); }
+void llama_get_logits(void) { absent("llama_get_logits"); }
+void llama_get_state_size(void) { absent("llama_get_state_size"); }
+void llama_init_candidates(void) { absent("llama_init_candidates"); }
+void llama_init_from_file(void) { absent("llama_init_from_file"); }
+void llama_load_session_file(void) { absent("llama_load_session_file"); }
+void llama_mlock_supported(void) { absent("llama_mlock_supported"); }
+void llama_mmap_supported(void) { absent("llama_mmap_supported"); }
+void llama_model_quantize(void) { absent("llama_model_quantize"); }
+void llama_n_ctx(void) { absent("llama_n_ctx"); }
+void llama_n_embd(void) { absent("llama_n_embd"); }
+void llama_n_vocab(void) { absent("llama_n_vocab"); }
+void llama_print_system_info(void) { absent("llama_print_system_info"); }
+void llama_print_timings(void) { absent("llama_print_timings"); }
+void llama_reset_timings(void) { absent("llama_reset_timings"); }
+void llama_sample_frequency_and_presence_penalties(void) { absent("llama_sample_frequency_and_presence_penalties"); }
+void llama_sample_repetition_penalty(void) { absent("llama_sample_repetition_penalty"); }
+void llama_sample_softmax(void) { absent("llama_sample_softmax"); }
+void llama_sample_tail_free(void) { absent("llama_sample_tail_free"); }
+void llama_sample_temperature(void) { absent("llama_sample_temperature"); }
+void llama_sample_token(void) { absent("llama_sample_token"); }
+void llama_sample_token_greedy(void) { absent("llama_sample_token_greedy"); }
+void llama_sample_token_mirostat(void) { absent("llama_sample_token_mirostat"); }
+void llama_sample_token_mirostat_v2(void) { absent("llama_sample_token_mirostat_v2"); }
+void llama_sample_top_k(void) { absent("llama_sample_top_k"); }
+void llama_sample_top_p(void) { absent("llama_sample_top_p"); }
+void llama_sample_typical(void) { absent("llama_sample_typical"); }
+void llama_save_session_file(void) { absent("llama_save_session_file"); }
+void llama_set_rng_seed(void) { absent("llama_set_rng_seed"); }
+void llama_set_state_data(void) { absent("llama_set_state_data"); }
+void llama_time_us(void) { absent("llama_time_us"); }
+void llama_token_bos(void) { absent("llama_token_bos"); }
+void llama_token_eos(void) { absent("llama_token_eos"); }
+void llama_token_nl(void) { absent("llama_token_nl"); }
+void llama_token_to_str(void) { absent("llama_token_to_str"); }
+void llama_tokenize(void) { absent("llama_tokenize"); }
+
 }  // extern "C"

@@ -174,3 +174,46 @@ def test_use_batch_forward_window():
 def test_real_quantization_without_a_gpu_fails_loudly():
     with pytest.raises(RuntimeError, match="MI355X|failed"):
         ggml_convert_qtype(torch.zeros(2, 64), Q["sym_int4"], device="cpu")
+
+
+# every name python/llm/src/ipex_llm/ggml/model/llama/llama_cpp.py resolves on the library at import
+# (`_lib.<name>.argtypes = ...` / `.restype = ...`, lines 228-1193): a missing one raises AttributeError there
+REFERENCE_IMPORT_SYMBOLS = [
+    "ggml_quantize_tensor", "ggml_quantize_tensor_with_weights", "ggml_quantize_tensor_rtn",
+    "ggml_quantize_tensor_rtn_with_weights", "ggml_type_size", "ggml_qk_size", "ggml_dequantize_q4_0",
+    "ggml_quantize_q4_0", "ggml_dequantize", "ggml_q_format_convet_cpu2xpu", "ggml_q_format_convet_xpu2cpu",
+    "ggml_compute_forward_mul_mat_q_fp32", "llama_init_backend",
+    "llama_apply_lora_from_file", "llama_context_default_params", "llama_copy_state_data", "llama_eval",
+    "llama_free", "llama_get_embeddings", "llama_get_kv_cache_token_count", "llama_get_logits",
+    "llama_get_state_size", "llama_init_candidates", "llama_init_from_file", "llama_load_session_file",
+    "llama_mlock_supported", "llama_mmap_supported", "llama_model_quantize", "llama_n_ctx", "llama_n_embd",
+    "llama_n_vocab", "llama_print_system_info", "llama_print_timings", "llama_reset_timings",
+    "llama_sample_frequency_and_presence_penalties", "llama_sample_repetition_penalty", "llama_sample_softmax",
+    "llama_sample_tail_free", "llama_sample_temperature", "llama_sample_token", "llama_sample_token_greedy",
+    "llama_sample_token_mirostat", "llama_sample_token_mirostat_v2", "llama_sample_top_k", "llama_sample_top_p",
+    "llama_sample_typical", "llama_save_session_file", "llama_set_rng_seed", "llama_set_state_data",
+    "llama_time_us", "llama_token_bos", "llama_token_eos", "llama_token_nl", "llama_token_to_str",
+    "llama_tokenize",
+]
+
+
+def test_library_exports_every_symbol_the_reference_resolves_at_import():
+    assert len(set(REFERENCE_IMPORT_SYMBOLS)) == 55
+    lib = ctypes.CDLL(os.path.join(ROOT, "ipex-llm_amd", "ipex_llm", "libs", "liblowbit_hip.so"))
+    for n in REFERENCE_IMPORT_SYMBOLS:
+        assert hasattr(lib, n), n
+
+
+def test_quantizers_outside_the_path_fail_with_a_message():
+    lib = ctypes.CDLL(os.path.join(ROOT, "ipex-llm_amd", "ipex_llm", "libs", "liblowbit_hip.so"))
+    lib.lowbit_last_error.restype = ctypes.c_char_p
+    lib.ggml_quantize_tensor_with_weights.restype = ctypes.c_size_t
+    lib.ggml_quantize_tensor_with_weights.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                                      ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    assert lib.ggml_quantize_tensor_with_weights(None, None, Q["q4_k"], 1, 256, None, None) == 0
+    assert b"not implemented" in lib.lowbit_last_error()
+    lib.ggml_quantize_tensor_rtn.restype = ctypes.c_size_t
+    lib.ggml_quantize_tensor_rtn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                             ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p, ctypes.c_bool]
+    assert lib.ggml_quantize_tensor_rtn(None, None, None, 2, 4096, 64, None, False) == 0
+    assert b"NPU" in lib.lowbit_last_error()
