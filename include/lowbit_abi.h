@@ -72,7 +72,8 @@ const char *lowbit_last_error(void);
 
 /* llama_cpp.py:946-967; called from low_bit_linear.py:162.  n = number of weights, k = row
  * length.  hist is ignored (the reference never reads it back, low_bit_linear.py:145);
- * scale_search = true is not implemented and fails.  Returns bytes written, 0 on failure. */
+ * scale_search = true (the closed binary's search for a better block scale) is not implemented: the
+ * plain block scale is used and a warning goes to stderr once.  Returns bytes written, 0 on failure. */
 size_t ggml_quantize_tensor(const float *src, void *dst, int qtype, size_t n, int k, int64_t *hist,
                             bool scale_search);
 /* llama_cpp.py:1050-1056 and :1059-1065.  0 for a qtype this library does not implement. */

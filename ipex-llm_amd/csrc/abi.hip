@@ -361,7 +361,16 @@ size_t ggml_quantize_tensor(const float *src, void *dst, int qtype, size_t n, in
                             bool scale_search) {
     (void)hist;
     g_err[0] = 0;
-    if (scale_search) { fail(LOWBIT_EARG, "ggml_quantize_tensor: scale_search is not implemented"); return 0; }
+    if (scale_search) {
+        // The search lives in the reference's closed binary and cannot be reproduced.  Its Python caller
+        // ignores the return value (low_bit_linear.py:162), so refusing would leave an uninitialised blob
+        // in a model: quantize with the plain absmax scale instead and say so once.
+        static bool warned = false;
+        if (!warned) {
+            warned = true;
+            fprintf(stderr, "liblowbit_hip: ggml_quantize_tensor: scale_search is not implemented; using the plain block scale\n");
+        }
+    }
     const int qk = qk_size(qtype);
     if (!qk) { fail(LOWBIT_EQTYPE, "ggml_quantize_tensor: unsupported qtype %d", qtype); return 0; }
     if (k <= 0 || k % qk || n % (size_t)k) { fail(LOWBIT_ESHAPE, "ggml_quantize_tensor: bad n/k"); return 0; }
