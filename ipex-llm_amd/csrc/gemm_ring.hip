@@ -352,17 +352,12 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
             set_tile(f_tile);                        // one tile past the end at worst: clamped, never fetched
         }
     };
-    auto issue_next = [&](int slot) {
-        issue(f_kt, slot);
-        if (++f_kt == G) {
-            f_kt = 0;
-            f_tile++;
-            set_tile(f_tile);                        // one tile past the end at worst: clamped, never fetched
-        }
-    };
 #pragma unroll
     for (int s = 0; s < S - 1; s++)
-        if (s < n_units) issue_next(s);
+        if (s < n_units) {
+            issue(f_kt, s);
+            fetched();
+        }
     int slot = 0, fill = S - 1;                      // slot of the current unit / of the next one to fill
     int c_tile = first_tile, c_kt = u0 - first_tile * G;
     WRegs wr;
