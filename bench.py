@@ -363,7 +363,7 @@ QT_BYTES = {2: (18, 32), 3: (20, 32), 8: (34, 32), 10: (34, 64), 15: (132, 128)}
 
 def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream):
     """The parity-test configurations of BASELINE.json timed once each (not the headline):
-    configs[2] prefill, configs[3] Llama-3-70B shapes in nf4 / sym_int8, configs[4] Mixtral experts."""
+    configs[2] prefill, configs[3] Llama-3-70B shapes in nf4 / sym_int8, configs[4] Mixtral experts (prefill and decode)."""
     res = {}
 
     def new_weight(n, k, qtype, std):
@@ -447,6 +447,26 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream):
     res["mixtral_moe_fp8_512tok_top2"] = {"ms": round(ms, 4), "TFLOP/s": round(flop / ms / 1e9, 1),
                                           "weight_GB/s": round(wb / ms / 1e6, 1),
                                           "rows_per_expert": [int(v) for v in (offsets[1:] - offsets[:-1]).tolist()]}
+    # the same experts at decode: one token through its top-2 experts in two launches (xe_linear.moe_forward_vec);
+    # 16 different expert pairs per graph replay, so that the weights come from HBM
+    pairs = [(i % n_exp, (i * 3 + 1) % n_exp) for i in range(16)]
+    ids = [torch.tensor(p, dtype=torch.int32, device=dev) for p in pairs]
+    rw = torch.tensor([0.6, 0.4], dtype=torch.float32, device=dev)
+    x1 = torch.randn((1, hid), generator=gen, device=dev).bfloat16()
+    work = torch.empty((2, ffn), dtype=torch.bfloat16, device=dev)
+    y1 = torch.empty((1, hid), dtype=torch.bfloat16, device=dev)
+
+    def moe_decode():
+        st = stream()
+        for t in ids:
+            ggml.lowbit_moe_forward(x1.data_ptr(), t.data_ptr(), rw.data_ptr(), 2, n_exp, ptrs["w1"].data_ptr(),
+                                    ptrs["w3"].data_ptr(), ptrs["w2"].data_ptr(), work.data_ptr(), y1.data_ptr(), qt,
+                                    ggml.DT_BF16, hid, ffn, 0, st)
+    g = capture(moe_decode)
+    ms = time_graph(g, 10, 2) / len(ids)
+    tok_bytes = 2 * 3 * blobs["w1"][0].numel()
+    res["mixtral_moe_fp8_decode_top2"] = {"ms": round(ms, 4), "weight_GB/s": round(tok_bytes / ms / 1e6, 1),
+                                          "launches_per_token": 2}
     return res
 
 
