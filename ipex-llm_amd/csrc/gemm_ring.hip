@@ -485,10 +485,9 @@ double ring_time_us(int M, int N, int K, int qtype, bool have_ws) {
     return fixed[i] - (p.ws_bytes ? 0.0 : 4.5) + run * step[i] * bytes * busy;
 }
 
-// enough for either tile width
+// every format runs 32 weight rows per wave (ring_rnb), so one plan covers them all
 size_t ring_workspace_bytes(int M, int N, int K, int wgs) {
-    const size_t a = ring_plan(M, N, K, 1, wgs, true).ws_bytes, b = ring_plan(M, N, K, 2, wgs, true).ws_bytes;
-    return a > b ? a : b;
+    return ring_plan(M, N, K, 1, wgs, true).ws_bytes;
 }
 
 template <int QT, typename AT, int MB, int RNB>
