@@ -216,6 +216,19 @@ int lowbit_forward_ws(const void *x, const void *w, void *y, int qtype, int layo
 int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
                    int64_t K, void *workspace, size_t workspace_bytes, int splits, void *stream);
 
+/* lowbit_forward_ws without a workspace argument and without any allocation: the partial tiles go to a
+ * scratch array that is part of the library's image on every GPU (lowbit_noalloc_scratch_bytes() = 64 MiB,
+ * held by each GPU the library runs on until the process ends).  No counterpart in the reference; it is for
+ * callers that cannot allocate device memory: code under HIP-graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  Same result as lowbit_forward_ws given lowbit_workspace_bytes(M, N, K) bytes; a
+ * shape that asks for more than the scratch holds fails with LOWBIT_ESIZE.  The call neither allocates nor
+ * frees (the scratch address is looked up once per device: by llama_init_backend for device 0, by the first
+ * call made with another device current for that device).  All calls on one GPU share the array: calls that
+ * overlap in time on one GPU (two streams) race on it - serialize them or use lowbit_forward_ws. */
+size_t lowbit_noalloc_scratch_bytes(void);
+int lowbit_forward_noalloc(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                           int64_t N, int64_t K, void *stream);
+
 /* The kernel lowbit_forward_ws picks for M of a few dozen to a few hundred rows (tiled layout, y
  * 8-byte aligned): 128 / 64 / 32 rows of x by 256 weight rows per workgroup, the (tile, K-step) units
  * dealt out in equal runs over `wgs` workgroups (0 = the library's choice), partial tiles summed from

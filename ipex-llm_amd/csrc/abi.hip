@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 namespace lowbit {
 int launch_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, void *out, int qtype, int64_t N,
                            int64_t K, int layout, int out_dtype, hipStream_t st);
@@ -258,6 +260,56 @@ int lowbit_forward_ws(const void *x, const void *w, void *y, int qtype, int layo
     return forward_any(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace ? workspace_bytes : 0, stream);
 }
 
+// ---- lowbit_forward_noalloc: lowbit_forward_ws over a workspace that is part of the library's image.
+//
+// `scratch` is the HOST-side handle of a device array: host code never passes the name itself to a kernel
+// or a copy.  Its device address differs per GPU and is looked up once per device with that device current
+// (llama_init_backend does it for device 0, the first call on any other device for that one).
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)64 << 20;
+static __device__ __align__(256) uint8_t scratch[NOALLOC_SCRATCH_BYTES];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static void *g_scratch_ptr[NOALLOC_MAX_DEVICES];
+static std::mutex g_scratch_mu;
+
+// device address of `scratch` on the current device; nullptr (with the error text set) on failure
+static void *scratch_of_current_device(const char *what) {
+    int dev = -1;
+    if (check_hip(hipGetDevice(&dev), what)) return nullptr;
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) {
+        fail(LOWBIT_EHIP, "%s: device ordinal %d is beyond the %d this library keeps scratch for", what, dev,
+             NOALLOC_MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        if (check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+        if (!p || (((uintptr_t)p) & 255)) {
+            fail(LOWBIT_EHIP, "%s: scratch array resolved to a null or misaligned address", what);
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+
+size_t lowbit_noalloc_scratch_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
+
+int lowbit_forward_noalloc(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                           int64_t N, int64_t K, void *stream) {
+    const char *what = "lowbit_forward_noalloc";
+    // the same workspace lowbit_forward_ws would be given by a caller that follows lowbit_workspace_bytes
+    const size_t need = layout == LOWBIT_LAYOUT_TILED ? lowbit_workspace_bytes(M, N, K) : 0;
+    if (need > NOALLOC_SCRATCH_BYTES)
+        return fail(LOWBIT_ESIZE, "%s: [%lld x %lld] at M = %lld wants %zu bytes of workspace, the built-in scratch holds "
+                    "%zu; use lowbit_forward_ws with a caller-owned workspace", what, (long long)N, (long long)K,
+                    (long long)M, need, NOALLOC_SCRATCH_BYTES);
+    if (!need) return forward_any(x, w, y, qtype, layout, act_dtype, M, N, K, nullptr, 0, stream);
+    void *ws = scratch_of_current_device(what);
+    if (!ws) return LOWBIT_EHIP;
+    return forward_any(x, w, y, qtype, layout, act_dtype, M, N, K, ws, need, stream);
+}
+
 int lowbit_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, void *dst, int qtype, int64_t N,
                            int64_t K, int layout, int out_dtype, void *stream) {
     if (int rc = check_weight_shape("lowbit_dequantize_rows", qtype, N, K, layout)) return rc;
@@ -445,7 +497,8 @@ void llama_init_backend(void) {
     int n = 0;
     if (check_hip(hipGetDeviceCount(&n), "hipGetDeviceCount")) return;
     if (n < 1) { fail(LOWBIT_EHIP, "llama_init_backend: no HIP device"); return; }
-    (void)check_hip(hipSetDevice(0), "hipSetDevice");
+    if (check_hip(hipSetDevice(0), "hipSetDevice")) return;
+    (void)scratch_of_current_device("llama_init_backend");      // device 0's address of the no-alloc scratch
 }
 
 

@@ -208,6 +208,21 @@ def lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, work
                                  stream), "lowbit_gemm_ring")
 
 
+_lib.lowbit_noalloc_scratch_bytes.argtypes = []
+_lib.lowbit_noalloc_scratch_bytes.restype = c_size_t
+_lib.lowbit_forward_noalloc.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
+                                        c_void_p]
+_lib.lowbit_forward_noalloc.restype = c_int
+
+
+def lowbit_noalloc_scratch_bytes() -> int:
+    return _lib.lowbit_noalloc_scratch_bytes()
+
+
+def lowbit_forward_noalloc(x, w, y, qtype, layout, act_dtype, m, n, k, stream):
+    _check(_lib.lowbit_forward_noalloc(x, w, y, qtype, layout, act_dtype, m, n, k, stream), "lowbit_forward_noalloc")
+
+
 _lib.lowbit_grouped_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int,
                                         c_int64, c_int64, c_void_p]
 _lib.lowbit_grouped_forward.restype = c_int
