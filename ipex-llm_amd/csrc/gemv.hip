@@ -434,7 +434,14 @@ static int launch_gemv_t(const void *x, const void *w, void *y, int layout, int 
                     if (mc <= 2) launch_mfma<QT, AT, 1, 2, 1>(xp, wp, yp, mc, N, K, waves, st);
                     else launch_mfma<QT, AT, 1, 2, 2>(xp, wp, yp, mc, N, K, waves, st);
                 }
-            } else if (mc <= 8) launch_mfma<QT, AT, 2, 4, 8>(xp, wp, yp, mc, N, K, waves, st);
+            }
+            // 5 .. 8 rows: one tile per wave and round with up to 16 waves keeps the x slice of a wave (and with
+            // it the workgroup's LDS footprint) small; two tile rows share x where N leaves enough workgroups
+            // (measured on MI355X, sym_int4: 5-7 % on the Llama-2-7B shapes, 15-20 % on [28672 x 8192] and
+            // [8192 x 28672] against four tiles per wave)
+            else if (mc <= 8 && (N / TILE_ROWS) % 2 == 0 && N >= 8192)
+                launch_mfma<QT, AT, 2, 1, 2, false, 0, 2>(xp, wp, yp, mc, N, K, waves, st);
+            else if (mc <= 8) launch_mfma<QT, AT, 2, 1, 2>(xp, wp, yp, mc, N, K, waves, st);
             // 9 .. 16 rows of x: share x between 4 or 2 tile rows where N still gives enough workgroups
             // (measured on MI355X: +25 .. 70 % on [28672 x 8192], +8 .. 24 % on [8192 x 8192])
             else if ((N / TILE_ROWS) % 4 == 0 && N >= 16384)
@@ -464,13 +471,14 @@ static int launch_gemv_q(const void *x, const void *w, void *y, int layout, int 
 template <int QT, typename AT>
 static int launch_mlp_t(const void *x, const void *wg, const void *wu, void *y, int M, int N, int K, int act,
                         hipStream_t st) {
-    // four tiles of each weight per wave and round, 8 waves for K = 4096: measured equal to two
-    // tiles with twice the rounds and ahead of 16-wave workgroups, which pack badly onto a CU
+    // Two tiles of each weight per wave and round, at most 8 waves: the registers of four tiles in flight
+    // keep the kernel below 80 vector registers, so that a CU holds three workgroups and the 688 workgroups
+    // of a [11008 x 4096] pair all run side by side.  With four tiles of each weight the kernel takes 120
+    // registers and a third of the workgroups has to wait for a free slot.
     const AT *xp = (const AT *)x;
     const uint8_t *g = (const uint8_t *)wg, *u = (const uint8_t *)wu;
-    if (M == 1) launch_mfma<QT, AT, 1, 4, 1, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
-    else if (M == 2) launch_mfma<QT, AT, 1, 4, 2, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
-    else launch_mfma<QT, AT, 1, 4, 4, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
+    if (M <= 2) launch_mfma<QT, AT, 1, 2, 1, true>(xp, g, (AT *)y, M, N, K, 8, st, u, act);
+    else launch_mfma<QT, AT, 1, 2, 2, true>(xp, g, (AT *)y, M, N, K, 8, st, u, act);
     return 0;
 }
 
