@@ -183,6 +183,9 @@ def _replace_with_low_bit_linear(model, qtype, modules_to_not_convert=None,
                 cur_qtype, cur_imatrix = get_cur_qtype_and_imatrix(qtype, full_module_name,
                                                                    imatrix_data, model_config)
                 cur_qtype = check_hidden_size(cur_qtype, in_features)
+                from ipex_llm.transformers.low_bit_linear import get_qk_size
+                if get_qk_size(cur_qtype) and in_features % get_qk_size(cur_qtype) != 0:
+                    continue   # rows that do not divide into blocks (fp8_e4m3: 128 weights) stay dense
                 with _empty_init():
                     new_linear = LowBitLinear(in_features, out_features, cur_qtype,
                                               module.bias is not None, mp_group=mp_group,
@@ -238,17 +241,28 @@ def _replace_with_low_bit_linear(model, qtype, modules_to_not_convert=None,
     return model, has_been_replaced
 
 
+# model types whose attention modules hold q_proj / k_proj / v_proj and get them merged by the reference's
+# _optimize_pre (convert.py:954-1008)
+_MERGE_QKV_MODEL_TYPES = ("llama", "mistral", "qwen2", "gemma", "gemma2", "minicpm", "stablelm", "mllama")
+
+
 def _optimize_pre(model, qtype=None):
-    return model    # q/k/v merging and friends: attention path, not built here
-
-
-def convert_forward(m, target_m, new_forward):
-    """Bind new_forward to every sub-module of class target_m (convert.py:1185-1193 of the reference)."""
-    from types import MethodType
-    if m.__class__ == target_m:
-        m.forward = MethodType(new_forward, m)
-    for _, sub_m in m.named_children():
-        convert_forward(sub_m, target_m, new_forward)
+    """Of the reference's pre-conversion passes (convert.py:880-1076) the one that belongs to the linear
+    path: q_proj / k_proj / v_proj become one `qkv_proj`, so that a decode step streams them in one launch
+    (convert.py:996-999 for Llama; the merge itself is models/common.py:40-52).  GPTQ checkpoints are left
+    alone, as in the reference (convert.py:954-960)."""
+    config = getattr(model, "config", None)
+    model_type = getattr(config, "model_type", None)
+    if model_type not in _MERGE_QKV_MODEL_TYPES:
+        return model
+    qcfg = getattr(config, "quantization_config", None)
+    if (qcfg.get("quant_method") if isinstance(qcfg, dict) else getattr(qcfg, "quant_method", None)) == "gptq":
+        return model
+    from ipex_llm.transformers.models.common import merge_qkv_base
+    for module in list(model.modules()):
+        if module.__class__.__name__.endswith("Attention"):
+            merge_qkv_base(module, module.__class__)
+    return model
 
 
 def _optimize_post(model):

@@ -217,3 +217,49 @@ def test_quantizers_outside_the_path_fail_with_a_message():
                                              ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p, ctypes.c_bool]
     assert lib.ggml_quantize_tensor_rtn(None, None, None, 2, 4096, 64, None, False) == 0
     assert b"NPU" in lib.lowbit_last_error()
+
+
+def test_optimize_pre_merges_qkv_and_the_stock_attention_forward_still_works():
+    """convert.py:996-999 / models/common.py:40-52 of the reference: q_proj, k_proj, v_proj become qkv_proj.
+    Dense weights on the CPU here (the merge happens before quantization)."""
+    transformers = pytest.importorskip("transformers")
+    from ipex_llm.transformers.convert import _optimize_pre
+    from ipex_llm.transformers.models.common import MergedProjectionSlice
+    cfg = transformers.LlamaConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=50,
+                                   max_position_embeddings=32)
+    torch.manual_seed(3)
+    model = transformers.LlamaForCausalLM(cfg).eval()
+    attn = model.model.layers[0].self_attn
+    wq, wk, wv = (getattr(attn, n).weight.detach().clone() for n in ("q_proj", "k_proj", "v_proj"))
+    ids = torch.randint(0, 50, (2, 7))
+    with torch.no_grad():
+        want = model(ids).logits
+    n_params = sum(p.numel() for p in model.parameters())
+    model = _optimize_pre(model)
+    attn = model.model.layers[0].self_attn
+    assert torch.equal(attn.qkv_proj.weight, torch.cat([wq, wk, wv]))
+    assert (attn.qkv_proj.in_features, attn.qkv_proj.out_features) == (64, 64 + 32 + 32)
+    assert all(isinstance(getattr(attn, n), MergedProjectionSlice) for n in ("q_proj", "k_proj", "v_proj"))
+    assert (attn.k_proj.start, attn.k_proj.length, attn.v_proj.start) == (64, 32, 96)
+    assert sum(p.numel() for p in model.parameters()) == n_params          # nothing is held twice
+    assert not any("q_proj" in k for k in model.state_dict())
+    with torch.no_grad():
+        got = model(ids).logits
+    assert torch.allclose(got, want, atol=1e-5, rtol=1e-5)
+    # a slice called on a tensor the merged product was not run on computes its own rows
+    x = torch.randn(3, 64)
+    assert torch.allclose(attn.v_proj(x), x @ wv.t(), atol=1e-5)
+    # merging twice changes nothing; other model types are left alone
+    again = _optimize_pre(model)
+    assert again.model.layers[0].self_attn.qkv_proj is attn.qkv_proj
+    gpt = transformers.GPT2LMHeadModel(transformers.GPT2Config(n_layer=1, n_head=2, n_embd=32, vocab_size=40))
+    assert _optimize_pre(gpt) is gpt
+
+
+def test_linears_whose_row_length_is_no_multiple_of_the_block_stay_dense():
+    # fp8_e4m3 blocks hold 128 weights: 192 input features pass the reference's % 64 rule but cannot be quantized
+    with torch.device("meta"):
+        m = nn.Sequential(nn.Linear(192, 64), nn.Linear(256, 64))
+    m, replaced = _replace_with_low_bit_linear(m, Q["fp8_e4m3"], convert_shape_only=True)
+    assert replaced and type(m[0]) is nn.Linear and isinstance(m[1], LowBitLinear)

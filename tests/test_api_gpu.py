@@ -182,6 +182,9 @@ def test_from_pretrained_tiny_llama_and_low_bit_round_trip(tmp_path):
     lin = model.model.layers[0].mlp.gate_proj
     assert isinstance(lin, LowBitLinear) and lin.weight.quantized
     assert type(model.lm_head) is nn.Linear
+    # q_proj / k_proj / v_proj were merged before quantization, as the reference does for Llama
+    attn = model.model.layers[0].self_attn
+    assert isinstance(attn.qkv_proj, LowBitLinear) and attn.qkv_proj.out_len == 3 * 128
     ids = torch.randint(0, 320, (1, 9))
     with torch.no_grad():
         want = hf(ids).logits

@@ -162,3 +162,54 @@ def test_from_pretrained_with_embedding_qtype_and_fused_mlp(tmp_path):
     with torch.no_grad():
         got2 = again.to("cuda")(ids.cuda()).logits.float().cpu()
     assert torch.equal(got, got2)
+
+
+# ------------------------------------------------------------------ merged q/k/v projection
+
+@pytest.mark.parametrize("qname,dtype", [("sym_int4", torch.float16), ("nf4", torch.bfloat16), ("sym_int8", torch.bfloat16)])
+@pytest.mark.parametrize("m", [1, 4, 40])
+def test_merged_qkv_projection_equals_the_three_separate_ones(qname, dtype, m):
+    """The merge of q_proj / k_proj / v_proj (convert.py:996-999 of the reference) is a row concatenation
+    before quantization; blocks never straddle rows, so the merged blob is the concatenation of the three
+    blobs and every output column must come out as from the separate layers: against the oracle on the
+    separate weights, and bit for bit where both calls run the same kernel variant."""
+    from ipex_llm.transformers.models.common import merge_qkv_base
+    qtype = Q[qname]
+    hidden, nq, nkv = 1024, 1024, 256
+
+    class Attention(nn.Module):                      # q/k/v as in a grouped-query attention block
+        def __init__(self):
+            super().__init__()
+            self.q_proj = nn.Linear(hidden, nq, bias=False)
+            self.k_proj = nn.Linear(hidden, nkv, bias=False)
+            self.v_proj = nn.Linear(hidden, nkv, bias=False)
+
+    torch.manual_seed(17)
+    attn = Attention().eval()
+    ws = [getattr(attn, n).weight.detach().clone() for n in ("q_proj", "k_proj", "v_proj")]
+    separate = []
+    for w in ws:
+        lin = LowBitLinear(hidden, w.shape[0], qtype, bias=False).eval()
+        lin.weight = FP4Params(w.clone(), qtype=qtype).to("cuda")
+        separate.append(lin)
+    merge_qkv_base(attn, Attention)
+    merged = LowBitLinear(hidden, nq + 2 * nkv, qtype, bias=False).eval()
+    merged.weight = FP4Params(attn.qkv_proj.weight.detach().clone(), qtype=qtype).to("cuda")
+    attn.qkv_proj = merged
+    # bytes: merged blob == concatenated blobs (ggml layout, as saved)
+    cat = np.concatenate([orc.quantize(w.numpy(), qtype) for w in ws])
+    assert np.array_equal(merged.weight.to("cpu").data.view(torch.uint8).numpy(), cat)
+    x = acts(9900 + m, m, hidden, dtype).cuda()
+    with torch.no_grad():
+        q, k, v = attn.q_proj(x), attn.k_proj(x), attn.v_proj(x)          # one launch, two cache reads
+        sep = [lin(x) for lin in separate]
+        own_rows = attn.v_proj(x.clone())                                  # not the cached tensor: own rows only
+    tol = 2e-3 if dtype == torch.float16 else 8e-3
+    for got, lin_out, w in zip((q, k, v), sep, ws):
+        want = orc.mul_mat_exact(orc.quantize(w.numpy(), qtype), x.float().cpu().numpy(), w.shape, qtype)
+        assert np.abs(got.float().cpu().numpy() - want).max() <= tol * np.abs(want).max()
+        # same rows through a differently shaped launch: fp32 sums may be associated differently, the rounded
+        # results agree to the last place or two
+        diff = (got.float() - lin_out.float()).abs().max().item()
+        assert diff <= 2.0 ** (-9 if dtype == torch.float16 else -6) * lin_out.float().abs().max().item()
+    assert torch.equal(own_rows, sep[2])                                   # same shape, same kernel: bit for bit
