@@ -341,9 +341,13 @@ def convert_bigdl_other_module(model, dtype):
 
 
 def convert_forward(m, target_m, new_forward):
-    """Re-binds `forward` of every sub-module of class target_m (convert.py:1185-1193)."""
+    """Re-binds `forward` of every sub-module of class target_m (convert.py:1185-1193).  The forward it
+    replaces stays reachable as `_forward_before_fusion`: the fused MLP forwards call it whenever a call
+    cannot be fused, so that a class whose own forward does more than the plain gated product keeps doing it."""
     import types
     if m.__class__ == target_m:
+        if "_forward_before_fusion" not in m.__dict__:
+            m.__dict__["_forward_before_fusion"] = m.forward
         m.forward = types.MethodType(new_forward, m)
     for _, sub_m in m.named_children():
         convert_forward(sub_m, target_m, new_forward)

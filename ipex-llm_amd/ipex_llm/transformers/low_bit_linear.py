@@ -8,8 +8,10 @@ every byte of arithmetic is done by liblowbit_hip.so through its C ABI.
 Weight residency rule used throughout: a blob on the CPU is in the ggml layout
 (what the reference saves to disk); a blob on the GPU is in the device layout,
 i.e. 16x128 tiles whenever out_features % 16 == 0 and in_features % 128 == 0 and
-the ggml layout otherwise.  FP4Params.to() converts between the two, as the
-reference does with ggml_q_format_convet_cpu2xpu / _xpu2cpu.
+the ggml layout otherwise.  FP4Params enforces the rule on every way a blob can
+reach the GPU (to(), cuda(), construction from a blob that is already there) and
+converts back on the way to the CPU, as the reference does with
+ggml_q_format_convet_cpu2xpu / _xpu2cpu.
 """
 import ctypes
 import os
@@ -303,6 +305,17 @@ def mlp_forward_xpu(x: torch.Tensor, weight1: torch.Tensor, weight2: torch.Tenso
                       "mlp_forward_xpu expects x of shape [batch_size, state_size] on the GPU")
     invalidInputError(ggml.lowbit_tileable(qtype, output_size, state_size),
                       "mlp_forward_xpu needs output_size % 16 == 0 and state_size % 128 == 0")
+    invalidInputError(x.dtype in _DT, f"unsupported activation dtype {x.dtype}")
+    invalidInputError(batch_size <= 4, "mlp_forward_xpu serves at most 4 rows")
+    want = ggml.lowbit_blob_bytes(qtype, output_size * state_size)
+    for name, w in (("weight1", weight1), ("weight2", weight2)):
+        invalidInputError(isinstance(w, torch.Tensor) and w.device == x.device,
+                          f"mlp_forward_xpu: {name} must be a quantized blob on the same GPU as x")
+        invalidInputError(w.is_contiguous() and _as_u8(w).numel() == want,
+                          f"mlp_forward_xpu: {name} has {_as_u8(w).numel()} bytes, expected {want} for "
+                          f"[{output_size}, {state_size}]")
+        invalidInputError(getattr(w, "blob_layout", ggml.LAYOUT_TILED) == ggml.LAYOUT_TILED,
+                          f"mlp_forward_xpu: {name} is not in the tiled device layout")
     xc = (x if x.dtype != torch.float32 else x.half()).contiguous()
     y = torch.empty((batch_size, output_size), dtype=xc.dtype, device=x.device)
     with torch.cuda.device(x.device):
@@ -326,9 +339,16 @@ class FP4Params(torch.nn.Parameter):
                 qtype=None,
                 imatrix=None,
                 in_features=None,
-                enable_scale_search=False):
+                enable_scale_search=False,
+                blob_layout=None):
         if data is None:
             data = torch.empty(0)
+        if quantized and blob_layout is None and data.device.type == _ACCEL and _shape is not None \
+                and data.numel() and not convert_shape_only:
+            # A quantized blob handed to the constructor is in the ggml layout by contract (it is what CPU
+            # tensors and checkpoints hold).  One that already lives on the GPU is re-tiled here, so that no
+            # GPU-resident FP4Params ever holds a ggml blob of a tileable shape.
+            data = _relayout(data, qtype, _shape, ggml.LAYOUT_GGML)
         self = torch.Tensor._make_subclass(cls, data, requires_grad)
         self.data = data
         self.quantized = quantized
@@ -363,6 +383,8 @@ class FP4Params(torch.nn.Parameter):
                                            convert_shape_only=self.convert_shape_only,
                                            imatrix=self.imatrix, in_features=self.in_features,
                                            enable_scale_search=self.enable_scale_search)
+            if self.data.device.type == _ACCEL:
+                self.data = _relayout(self.data, qtype, w.shape, ggml.LAYOUT_GGML)   # residency rule
             self.quantized = True
             self._shape = w.shape
         return self
@@ -370,10 +392,34 @@ class FP4Params(torch.nn.Parameter):
     def get_shape(self):
         return self._shape
 
+    @property
+    def blob_layout(self):
+        """Layout of the blob as it is held right now: ggml on the CPU / meta device, the device layout of
+        its shape on the GPU.  Derived, not stored: nn.Module._apply swaps `.data` under an existing
+        parameter object, which would leave a stored value behind."""
+        if not self.quantized or self.data.device.type != _ACCEL or self._shape is None:
+            return ggml.LAYOUT_GGML
+        return device_layout(self.qtype, self._shape)
+
     def _clone_with(self, data):
+        # `data` already obeys the residency rule: say so, or the constructor would re-tile it
         return FP4Params(data, requires_grad=self.requires_grad, quantized=self.quantized,
                          _shape=self._shape, qtype=self.qtype,
-                         enable_scale_search=self.enable_scale_search)
+                         enable_scale_search=self.enable_scale_search,
+                         blob_layout=device_layout(self.qtype, self._shape)
+                         if self.quantized and self._shape is not None and data.device.type == _ACCEL
+                         else ggml.LAYOUT_GGML)
+
+    def cuda(self, device=None, non_blocking=False, **kwargs):
+        # Tensor.cuda() would copy the bytes as they are: a ggml blob would land on the GPU untiled
+        if device is None:
+            device = torch.device(_ACCEL, torch.cuda.current_device())
+        elif isinstance(device, int):
+            device = torch.device(_ACCEL, device)
+        return self.to(device=device, non_blocking=non_blocking)
+
+    def cpu(self, **kwargs):
+        return self.to(device="cpu")
 
     def to(self, *args, **kwargs):
         device, dtype, non_blocking, _ = torch._C._nn._parse_to(*args, **kwargs)
@@ -434,7 +480,7 @@ class MatMulLowBit(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, A, weight, output_size):
-        result = forward_new(A, weight.data, weight.qtype, output_size)
+        result = forward_new(A, weight.data, weight.qtype, output_size, layout=weight.blob_layout)
         ctx.tensors = (A, weight) if any(ctx.needs_input_grad[:2]) else (None, None)
         return result
 
@@ -443,7 +489,7 @@ class MatMulLowBit(torch.autograd.Function):
         A, weight = ctx.tensors
         grad_A = None
         if ctx.needs_input_grad[0]:
-            dequant_weight = dequant(A, weight.data, weight.qtype, shape=weight._shape)
+            dequant_weight = dequant(A, weight.data, weight.qtype, layout=weight.blob_layout, shape=weight._shape)
             grad_A = torch.matmul(grad_output.to(A.dtype), dequant_weight.reshape(weight._shape))
         return grad_A, None, None
 
@@ -508,12 +554,13 @@ class LowBitLinear(nn.Linear):
                 if do_empty_cache:
                     torch.cuda.empty_cache()
                 w = self.weight.data
+                layout = self.weight.blob_layout
                 if use_batch_forward(x_2d, self.weight.qtype, self.out_len):
-                    result = batch_forward(x_2d, w, self.qtype, self.out_len)
+                    result = batch_forward(x_2d, w, self.qtype, self.out_len, layout=layout)
                 else:
                     # fp32 activations are computed in half precision, as the reference does
                     # for M > 1 (low_bit_linear.py:660-665); forward_new casts back
-                    result = forward_new(x_2d, w, self.qtype, self.out_len)
+                    result = forward_new(x_2d, w, self.qtype, self.out_len, layout=layout)
                 if do_empty_cache:
                     torch.cuda.empty_cache()
             result = result.view(new_shape)

@@ -72,7 +72,8 @@ def _project_rows(linear: torch.nn.Module, x: torch.Tensor, start: int, length: 
         blob = w.data.view(torch.uint8)
         row_bytes = blob.numel() // linear.out_len
         x_2d = x.contiguous().view(-1, x.shape[-1])
-        y = forward_new(x_2d, blob[start * row_bytes:(start + length) * row_bytes], w.qtype, length)
+        y = forward_new(x_2d, blob[start * row_bytes:(start + length) * row_bytes], w.qtype, length,
+                        layout=w.blob_layout)
         y = y.view(*x.shape[:-1], length)
         return y if bias is None else y + bias.to(y.dtype)
     return linear(x)[..., start:start + length]
@@ -109,6 +110,10 @@ def fuse_mlp_base(module: torch.nn.Module, act: int, x: torch.Tensor):
     qtype = getattr(gate, "qtype", None)
     fusable = (isinstance(gate, LowBitLinear) and isinstance(up, LowBitLinear)
                and gate.bias is None and up.bias is None
+               and gate.weight.quantized and up.weight.quantized
+               and gate.weight.data.device == x.device and up.weight.data.device == x.device
+               and gate.weight.blob_layout == ggml.LAYOUT_TILED and up.weight.blob_layout == ggml.LAYOUT_TILED
+               and gate.in_len == up.in_len == x.size(-1)
                and up.qtype == qtype and gate.out_len == up.out_len
                and x.dtype in (torch.float16, torch.bfloat16, torch.float32)
                and mlp_fusion_check(x, qtype, module.training)
@@ -119,6 +124,9 @@ def fuse_mlp_base(module: torch.nn.Module, act: int, x: torch.Tensor):
             mlp_forward_xpu(x_2d, gate.weight.data, up.weight.data, x_2d.size(0), x_2d.size(1), gate.out_len,
                             act, qtype))
         return output.view(*x.shape[:-1], output.size(-1))
+    original = module.__dict__.get("_forward_before_fusion")
+    if original is not None:
+        return original(x)                    # whatever this class does besides the plain gated product
     return module.down_proj(module.act_fn(module.gate_proj(x)) * module.up_proj(x))
 
 

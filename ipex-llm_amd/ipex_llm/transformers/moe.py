@@ -38,8 +38,21 @@ class ExpertWeights:
                               "experts must be quantized, on the GPU and of one shape / qtype")
         invalidInputError(ggml.lowbit_tileable(self.qtype, self.out_len, self.in_len),
                           "grouped experts need out_features % 16 == 0 and in_features % 128 == 0")
+        want = ggml.lowbit_blob_bytes(self.qtype, self.out_len * self.in_len)
+        for lin in linears:
+            invalidInputError(lin.weight.data.device == l0.weight.data.device
+                              and lin.weight.blob_layout == ggml.LAYOUT_TILED
+                              and _as_u8(lin.weight.data).numel() == want and lin.weight.data.is_contiguous(),
+                              "every expert must hold a tiled blob of the common shape on one GPU")
+        self.linears = list(linears)
         self.blobs = [_as_u8(lin.weight.data) for lin in linears]        # keeps the storage alive
         self.ptrs = torch.tensor([b.data_ptr() for b in self.blobs], dtype=torch.int64, device=l0.weight.device)
+
+    def check(self, device):
+        """The pointer table is a snapshot: refuse to launch if a layer was moved or re-quantized since."""
+        for lin, blob in zip(self.linears, self.blobs):
+            invalidInputError(lin.weight.data.data_ptr() == blob.data_ptr() and blob.device == device,
+                              "an expert weight was moved or replaced after ExpertWeights was built; build it again")
 
 
 def grouped_forward(x_sorted: torch.Tensor, group_offsets: torch.Tensor, experts: ExpertWeights):
@@ -48,6 +61,7 @@ def grouped_forward(x_sorted: torch.Tensor, group_offsets: torch.Tensor, experts
                       and x_sorted.dtype != torch.float32, "x must be [rows, K] in fp16 / bf16")
     invalidInputError(group_offsets.dtype == torch.int32 and group_offsets.numel() == len(experts.blobs) + 1
                       and group_offsets.device == x_sorted.device, "group_offsets must be int32 [E + 1] on the GPU")
+    experts.check(x_sorted.device)
     x_sorted = x_sorted.contiguous()
     rows = x_sorted.shape[0]
     y = torch.empty((rows, experts.out_len), dtype=x_sorted.dtype, device=x_sorted.device)
@@ -70,6 +84,8 @@ def moe_forward_vec(x: torch.Tensor, topk_ids: torch.Tensor, topk_weight: torch.
     invalidInputError((ups.qtype, ups.out_len, ups.in_len) == (gates.qtype, inter, hidden)
                       and (downs.qtype, downs.out_len, downs.in_len) == (gates.qtype, hidden, inter),
                       "gate / up / down experts do not fit together")
+    for table in (gates, ups, downs):
+        table.check(x.device)
     top_k = topk_ids.numel()
     ids = topk_ids.reshape(-1).to(torch.int32)
     rw = topk_weight.reshape(-1).to(torch.float32)

@@ -263,3 +263,37 @@ def test_linears_whose_row_length_is_no_multiple_of_the_block_stay_dense():
         m = nn.Sequential(nn.Linear(192, 64), nn.Linear(256, 64))
     m, replaced = _replace_with_low_bit_linear(m, Q["fp8_e4m3"], convert_shape_only=True)
     assert replaced and type(m[0]) is nn.Linear and isinstance(m[1], LowBitLinear)
+
+
+def test_fused_mlp_refuses_weights_that_are_not_tiled_blobs_next_to_x():
+    """A raw pointer only reaches the fused gate/up kernel after the checks forward_new makes; anything else
+    takes the module's own forward."""
+    from ipex_llm.transformers.low_bit_linear import mlp_forward_xpu
+    from ipex_llm.transformers.models.common import fuse_mlp_base
+    x = torch.zeros(1, 128, dtype=torch.half)
+    blob = torch.zeros(64 * 128 // 32 * 18, dtype=torch.uint8)
+    with pytest.raises(RuntimeError, match="GPU"):
+        mlp_forward_xpu(x, blob, blob, 1, 128, 64, 0, 2)                  # x on the CPU
+
+    class Mlp(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate_proj = nn.Linear(128, 64, bias=False)
+            self.up_proj = nn.Linear(128, 64, bias=False)
+            self.down_proj = nn.Linear(64, 128, bias=False)
+            self.act_fn = nn.SiLU()
+            self.calls = 0
+
+        def forward(self, x):
+            self.calls += 1
+            return 2.0 * self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))   # not the plain form
+
+    from ipex_llm.transformers.convert import convert_forward
+    from ipex_llm.transformers.models.common import mlp_silu_forward
+    m = Mlp().eval()
+    xf = torch.randn(2, 128)
+    want = m(xf)
+    convert_forward(m, Mlp, mlp_silu_forward)
+    got = m(xf)                                                           # dense CPU weights: cannot be fused
+    assert torch.equal(got, want) and m.calls == 2                        # the class's own forward ran
+    assert fuse_mlp_base(m, 0, xf).shape == (2, 128)

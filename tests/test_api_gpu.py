@@ -249,3 +249,34 @@ def test_lowbit_linears_replay_correctly_from_a_hip_graph():
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(static_y, want), (rows, step)
+
+
+@pytest.mark.parametrize("qname", ["sym_int4", "nf4"])
+def test_module_cuda_and_cpu_keep_the_residency_rule(qname):
+    """model.cuda() calls Tensor.cuda on every parameter, not .to(): the blob must still arrive tiled, and
+    model.cpu() must bring the ggml bytes back."""
+    qtype = Q[qname]
+    torch.manual_seed(21)
+    w = torch.randn(64, 256) * 0.02
+    lin = LowBitLinear(256, 64, qtype, bias=False).eval()
+    lin.weight = FP4Params(w.clone(), qtype=qtype)
+    net = nn.Sequential(lin).cuda()
+    p = net[0].weight
+    assert p.quantized and p.data.device.type == "cuda" and p.blob_layout == ggml.LAYOUT_TILED
+    blob = orc.quantize(w.numpy(), qtype)
+    x = torch.randn(5, 256).half()
+    y = net(x.cuda()).float().cpu().numpy()
+    want = orc.mul_mat_exact(blob, x.float().numpy(), (64, 256), qtype)
+    assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max()
+    # a quantized CPU blob through .cuda() as well (not only an unquantized weight)
+    back = net.cpu()
+    assert np.array_equal(back[0].weight.data.view(torch.uint8).numpy(), blob)
+    again = back.cuda()
+    assert np.array_equal(again(x.cuda()).float().cpu().numpy(), y)
+    # FP4Params built from a ggml blob that already lives on the GPU
+    born = FP4Params(torch.from_numpy(blob).cuda() if qname != "nf4" else torch.from_numpy(blob).cuda().view(torch.bfloat16),
+                     quantized=True, _shape=torch.Size((64, 256)), qtype=qtype)
+    assert torch.equal(born.data.view(torch.uint8), again[0].weight.data.view(torch.uint8))
+    # quantize(device) lands tiled too
+    direct = FP4Params(w.clone(), qtype=qtype).quantize("cuda")
+    assert torch.equal(direct.data.view(torch.uint8), born.data.view(torch.uint8))

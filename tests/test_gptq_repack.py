@@ -127,3 +127,29 @@ def test_converted_gptq_layer_runs_on_the_gpu():
     y = net.to("cuda").proj(x.cuda()).float().cpu().numpy()
     want = x.float().numpy() @ w.T.astype(np.float32) + bias
     assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max()
+
+
+@pytest.mark.gpu
+def test_gptq_layer_converted_while_already_on_the_gpu():
+    """The packed tensors of the source layer sit on the GPU, so the repacked blob is born there in the ggml
+    layout; the parameter has to re-tile it (nothing passes through FP4Params.to from the CPU here)."""
+    import lowbit_oracle as orc
+    from ipex_llm.transformers.low_bit_linear import LowBitLinear
+    import ipex_llm.ggml.model.llama.llama_cpp as ggml
+    q, zeros, scales = _case(6, in_f=256, out_f=64)
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.proj = FakeQuantLinear(q, zeros, scales, 128)
+    blob_cpu, _ = convert_gptq(FakeQuantLinear(q, zeros, scales, 128))
+    net, replaced = _replace_with_low_bit_linear(Net().to("cuda"), Q["asym_int4"])
+    assert replaced and isinstance(net.proj, LowBitLinear)
+    wp = net.proj.weight
+    assert wp.data.device.type == "cuda" and wp.blob_layout == ggml.LAYOUT_TILED
+    assert not torch.equal(wp.data.cpu(), blob_cpu)                       # tiled on the device ...
+    assert torch.equal(wp.to("cpu").data, blob_cpu)                        # ... the ggml bytes again on the host
+    x = torch.randn(3, 256).half()
+    y = net.proj(x.cuda()).float().cpu().numpy()
+    want = orc.mul_mat_exact(blob_cpu.numpy(), x.float().numpy(), (64, 256), Q["asym_int4"])
+    assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max()
