@@ -90,8 +90,9 @@ void ggml_dequantize(const void *src, void *dst, size_t k, int qtype);
 void ggml_q_format_convet_cpu2xpu(const void *src, void *dst, size_t n, int qtype);
 void ggml_q_format_convet_xpu2cpu(const void *src, void *dst, size_t n, int qtype);
 /* llama_cpp.py:1154-1185; called from low_bit_linear.py:487.  ne = {K, rows} (ggml order),
- * src0 = ggml blob [N, K], src1 = fp32 [M, K], dst = fp32 [M, N].  Activations are rounded to
- * fp16 on the device (the reference rounds them to int8 blocks instead). */
+ * src0 = ggml blob [N, K], src1 = fp32 [M, K], dst = fp32 [M, N].  Runs lowbit_forward_f32 on the device:
+ * activations keep 16 mantissa bits and fp32's range (the reference rounds them to int8 blocks), the
+ * result is never rounded to half precision. */
 void ggml_compute_forward_mul_mat_q_fp32(const int64_t *src0_ne, const void *src0, int qtype,
                                          const int64_t *src1_ne, const void *src1, void *dst);
 /* llama_cpp.py:1189-1193.  Selects device 0 and loads the kernels. */
@@ -215,6 +216,17 @@ int lowbit_forward_ws(const void *x, const void *w, void *y, int qtype, int layo
  * n * ceil(M/128) * ceil(N/256) * 128 KiB of workspace), 1 = none. */
 int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,
                    int64_t K, void *workspace, size_t workspace_bytes, int splits, void *stream);
+
+/* fp32 activations in, fp32 out: what xe_linear.forward_new / xe_batch.batch_forward compute when LowBitLinear
+ * hands them a float x (python/llm/src/ipex_llm/transformers/low_bit_linear.py:657-668: only M > 1 with
+ * conver_to_half casts to half first) and what the CPU branch's ggml_compute_forward_mul_mat_q_fp32 returns.
+ * x is split into two bf16 planes (16 mantissa bits, fp32's exponent range), the product of the 2M rows is
+ * accumulated and stored in fp32 and the halves are added.  The streaming kernel serves every M (16 rows of
+ * the planes per pass over the weights): meant for decode and small batches.  workspace: caller-owned device
+ * memory of lowbit_forward_f32_workspace_bytes(M, N, K) bytes, 16-byte aligned. */
+size_t lowbit_forward_f32_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int lowbit_forward_f32(const float *x, const void *w, float *y, int qtype, int layout, int64_t M, int64_t N, int64_t K,
+                       void *workspace, size_t workspace_bytes, void *stream);
 
 /* lowbit_forward_ws without a workspace argument and without any allocation: the partial tiles go to a
  * scratch array that is part of the library's image on every GPU (lowbit_noalloc_scratch_bytes() = 64 MiB,

@@ -30,6 +30,8 @@ int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, in
                 void *workspace, size_t workspace_bytes, int want_splits, hipStream_t st);
 int gemm_splits(int M, int N, int K, size_t ws_bytes);
 double gemm_time_us(int M, int N, int K, int splits);
+int launch_gemv_bf16_f32out(const void *x, const void *w, void *y, int qtype, int layout, int M, int N, int K,
+                            hipStream_t st);
 int launch_grouped_gemm(const void *x, const void *const *w, void *y, const int32_t *offsets, int n_groups,
                         int total_rows, int qtype, int act_dtype, int N, int K, hipStream_t st);
 }  // namespace lowbit
@@ -260,6 +262,57 @@ int lowbit_forward_ws(const void *x, const void *w, void *y, int qtype, int layo
     return forward_any(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace ? workspace_bytes : 0, stream);
 }
 
+// ---- lowbit_forward_f32: fp32 activations in, fp32 out
+//
+// The MFMA operands are 16-bit, so x is split into two bf16 planes, hi = bf16(x) and lo = bf16(x - hi)
+// (16 mantissa bits together, fp32's exponent range: no overflow whatever the magnitude of x), the product
+// runs on the 2M rows with fp32 output and the two halves are added.
+__global__ __launch_bounds__(256) void split_bf16_kernel(const float *__restrict__ x, __bf16 *__restrict__ hi,
+                                                         __bf16 *__restrict__ lo, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i];
+    const __bf16 h = (__bf16)v;                              // round to nearest even
+    const float r = v - (float)h;                            // exact: both share the leading bits
+    hi[i] = h;
+    lo[i] = (r == r && (r - r) == 0.0f) ? (__bf16)r : (__bf16)0.0f;   // inf / nan stay in the hi plane only
+}
+__global__ __launch_bounds__(256) void add_f32_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                      float *__restrict__ y, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = a[i] + b[i];
+}
+
+static size_t f32_plane_bytes(int64_t M, int64_t K) { return ((size_t)(2 * M * K * 2) + 255) & ~(size_t)255; }
+
+extern "C" size_t lowbit_forward_f32_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return f32_plane_bytes(M, K) + (size_t)(2 * M * N) * sizeof(float);
+}
+
+extern "C" int lowbit_forward_f32(const float *x, const void *w, float *y, int qtype, int layout, int64_t M, int64_t N,
+                                  int64_t K, void *workspace, size_t workspace_bytes, void *stream) {
+    const char *what = "lowbit_forward_f32";
+    if (int rc = check_weight_shape(what, qtype, N, K, layout)) return rc;
+    if (M < 0 || M > 0x3fffffff) return fail(LOWBIT_EARG, "%s: bad M", what);
+    if (M * N * K == 0) return 0;
+    if (!x || !w || !y || !aligned16(x) || !aligned16(w) || (((uintptr_t)y) & 3))
+        return fail(LOWBIT_EARG, "%s: null or misaligned pointer (x, w: 16 bytes)", what);
+    if (K % 8) return fail(LOWBIT_ESHAPE, "%s: K must be a multiple of 8", what);
+    const size_t need = lowbit_forward_f32_workspace_bytes(M, N, K);
+    if (!workspace || !aligned16(workspace) || workspace_bytes < need)
+        return fail(LOWBIT_ESIZE, "%s: needs %zu bytes of 16-byte aligned workspace", what, need);
+    hipStream_t st = (hipStream_t)stream;
+    __bf16 *planes = (__bf16 *)workspace;
+    float *y2 = (float *)((uint8_t *)workspace + f32_plane_bytes(M, K));
+    const int64_t nx = M * K, ny = M * N;
+    hipLaunchKernelGGL(split_bf16_kernel, dim3((unsigned)((nx + 255) / 256)), dim3(256), 0, st, x, planes, planes + nx, nx);
+    if (int rc = check_launch(launch_gemv_bf16_f32out(planes, w, y2, qtype, layout, (int)(2 * M), (int)N, (int)K, st), what))
+        return rc;
+    hipLaunchKernelGGL(add_f32_kernel, dim3((unsigned)((ny + 255) / 256)), dim3(256), 0, st, y2, y2 + ny, y, ny);
+    return check_hip(hipGetLastError(), what);
+}
+
 // ---- lowbit_forward_noalloc: lowbit_forward_ws over a workspace that is part of the library's image.
 //
 // `scratch` is the HOST-side handle of a device array: host code never passes the name itself to a kernel
@@ -374,15 +427,6 @@ int lowbit_grouped_forward(const void *x, const void *const *w, void *y, const i
 
 namespace {
 
-template <typename T> __global__ void cast_f32_kernel(const float *in, T *out, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = (T)in[i];
-}
-template <typename T> __global__ void cast_to_f32_kernel(const T *in, float *out, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = (float)in[i];
-}
-
 struct DevBuf {
     void *p = nullptr;
     ~DevBuf() { if (p) (void)hipFree(p); }
@@ -469,15 +513,12 @@ void ggml_compute_forward_mul_mat_q_fp32(const int64_t *src0_ne, const void *src
     if (M * N == 0) return;
     const size_t wbytes = lowbit_blob_bytes(qtype, N * K);
     const bool tile = lowbit_tileable(qtype, N, K);
-    DevBuf w, wt, xf, xh, yh, yf;
-    if (w.alloc(wbytes) || xf.alloc((size_t)M * K * 4) || xh.alloc((size_t)M * K * 2) ||
-        yh.alloc((size_t)M * N * 2) || yf.alloc((size_t)M * N * 4)) return;
+    const size_t ws_bytes = lowbit_forward_f32_workspace_bytes(M, N, K);
+    DevBuf w, wt, xf, ws, yf;
+    if (w.alloc(wbytes) || xf.alloc((size_t)M * K * 4) || ws.alloc(ws_bytes) || yf.alloc((size_t)M * N * 4)) return;
     if (tile && wt.alloc(wbytes)) return;
     if (check_hip(hipMemcpy(w.p, src0, wbytes, hipMemcpyHostToDevice), "hipMemcpy")) return;
     if (check_hip(hipMemcpy(xf.p, src1, (size_t)M * K * 4, hipMemcpyHostToDevice), "hipMemcpy")) return;
-    const int64_t nx = M * K, ny = M * N;
-    hipLaunchKernelGGL((cast_f32_kernel<_Float16>), dim3((unsigned)((nx + 255) / 256)), dim3(256), 0, nullptr,
-                       (const float *)xf.p, (_Float16 *)xh.p, nx);
     const void *wdev = w.p;
     int layout = LOWBIT_LAYOUT_GGML;
     if (tile) {
@@ -485,11 +526,9 @@ void ggml_compute_forward_mul_mat_q_fp32(const int64_t *src0_ne, const void *src
         wdev = wt.p;
         layout = LOWBIT_LAYOUT_TILED;
     }
-    if (lowbit_forward(xh.p, wdev, yh.p, qtype, layout, LOWBIT_DT_F16, M, N, K, nullptr)) return;
-    hipLaunchKernelGGL((cast_to_f32_kernel<_Float16>), dim3((unsigned)((ny + 255) / 256)), dim3(256), 0, nullptr,
-                       (const _Float16 *)yh.p, (float *)yf.p, ny);
-    if (check_hip(hipGetLastError(), "cast")) return;
-    (void)check_hip(hipMemcpy(dst, yf.p, (size_t)ny * 4, hipMemcpyDeviceToHost), "hipMemcpy");
+    // fp32 in, fp32 out, as the reference's CPU kernel: nothing is rounded to half precision on the way
+    if (lowbit_forward_f32((const float *)xf.p, wdev, (float *)yf.p, qtype, layout, M, N, K, ws.p, ws_bytes, nullptr)) return;
+    (void)check_hip(hipMemcpy(dst, yf.p, (size_t)M * N * 4, hipMemcpyDeviceToHost), "hipMemcpy");
 }
 
 void llama_init_backend(void) {

@@ -168,7 +168,10 @@ constexpr int GEMV_LDS_X_BUDGET = 64 * 1024;
 //   MOE == 2: x is the [slots, K / slots] output of the first launch, read as one long vector;
 //             tile g of the K walk belongs to slot g / ge and is scaled by route_w[slot]:
 //             y = sum_j route_w[j] * (x_j Wd[e_j]^T).
-template <int QT, typename AT, int MT, int U, int XN, bool DUAL, int MOE, int R>
+//
+// F32OUT: y is float [M, N] instead of AT (the fp32 path of lowbit_forward_f32: x arrives as two bf16 planes,
+// the sums must not be rounded to 8 bits on the way out).
+template <int QT, typename AT, int MT, int U, int XN, bool DUAL, int MOE, int R, bool F32OUT>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                          const uint8_t *__restrict__ w2, AT *__restrict__ y, int M,
                                                          int N, int K, int act, const int32_t *__restrict__ ids,
@@ -187,9 +190,15 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     // M = 16 a workgroup otherwise pulls 3.5 bytes of x out of L2 per byte of weight)
     constexpr int NW = DUAL ? 2 : R;
     static_assert(!(DUAL && R != 1) && XN * 1024 >= NW * MT * 256, "bad GEMV shape parameters");
-    __shared__ AT lut[16];
+    // nf4 code book in the activation type.  With fp32 output a second table holds what the rounding to AT
+    // dropped, and a second MFMA per sub-block adds it: the weights then carry 16 mantissa bits like x does.
+    __shared__ AT lut[16], lut_lo[16];
     if constexpr (QT == QT_NF4) {
-        if (threadIdx.x < 16) lut[threadIdx.x] = to_at<AT>(NF4_CODEBOOK[threadIdx.x]);
+        if (threadIdx.x < 16) {
+            const AT hi = to_at<AT>(NF4_CODEBOOK[threadIdx.x]);
+            lut[threadIdx.x] = hi;
+            lut_lo[threadIdx.x] = to_at<AT>(NF4_CODEBOOK[threadIdx.x] - (float)hi);
+        }
         __syncthreads();
     }
 
@@ -311,7 +320,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
                     }
                     d = live ? d : 0.0f;
                     mn = live ? mn : 0.0f;
-                    const f32x4 p = mfma16(a[j], b, zero4);
+                    f32x4 p = mfma16(a[j], b, zero4);
+                    if constexpr (QT == QT_NF4 && F32OUT) p = mfma16(a[j], Unpack<QT, AT>::run(tl.q0[j], lut_lo, magic), p);
                     if constexpr (NEED_S) {
                         const f32x4 s = mfma16(a[j], ones, zero4);
                         const float e = mn - OFFSET * d;
@@ -348,14 +358,19 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
                 s = gate_act(s, act) * u;
             }
             const int m = grp * MT + i;
-            if (m < M) y[(int64_t)m * N + ((int64_t)blockIdx.x * R + wave) * 16 + col] = to_at<AT>(s);
+            const int64_t at = (int64_t)m * N + ((int64_t)blockIdx.x * R + wave) * 16 + col;
+            if constexpr (F32OUT) {
+                if (m < M) ((float *)y)[at] = s;
+            } else {
+                if (m < M) y[at] = to_at<AT>(s);
+            }
         }
     }
 }
 
 // --------------------------------------------------------- generic GEMV
 
-template <int QT, int LAYOUT, typename AT, int MC>
+template <int QT, int LAYOUT, typename AT, int MC, bool F32OUT>
 __global__ __launch_bounds__(256) void gemv_generic_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                            AT *__restrict__ y, int m0, int M, int N, int K) {
     const int lane = threadIdx.x & 63;
@@ -387,13 +402,16 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const AT *__restrict_
     for (int mi = 0; mi < MC; mi++) {
         float v = acc[mi];
         for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-        if (lane == 0 && m0 + mi < M) y[(int64_t)(m0 + mi) * N + n] = to_at<AT>(v);
+        if (lane == 0 && m0 + mi < M) {
+            if constexpr (F32OUT) ((float *)y)[(int64_t)(m0 + mi) * N + n] = v;
+            else y[(int64_t)(m0 + mi) * N + n] = to_at<AT>(v);
+        }
     }
 }
 
 // -------------------------------------------------------------- launch
 
-template <int QT, typename AT, int MT, int U, int XN, bool DUAL = false, int MOE = 0, int R = 1>
+template <int QT, typename AT, int MT, int U, int XN, bool DUAL = false, int MOE = 0, int R = 1, bool F32OUT = false>
 static void launch_mfma(const AT *x, const uint8_t *w, AT *y, int M, int N, int K, int waves, hipStream_t st,
                         const uint8_t *w2 = nullptr, int act = 0, const int32_t *ids = nullptr,
                         const float *route_w = nullptr, int ge = 0, int slots = 1, int n_exp = 1) {
@@ -406,8 +424,32 @@ static void launch_mfma(const AT *x, const uint8_t *w, AT *y, int M, int N, int 
     if (waves > 0 && waves < wv) wv = waves;
     if (wv < 1) wv = 1;
     const size_t lds = (size_t)wv * XN * 512 * sizeof(AT);
-    hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, MT, U, XN, DUAL, MOE, R>), dim3(N / TILE_ROWS / R, MOE == 1 ? slots : 1),
+    hipLaunchKernelGGL((gemv_mfma_kernel<QT, AT, MT, U, XN, DUAL, MOE, R, F32OUT>), dim3(N / TILE_ROWS / R, MOE == 1 ? slots : 1),
                        dim3(64 * wv), lds, st, x, w, w2, y, M, N, K, act, ids, route_w, ge, n_exp);
+}
+
+// y in fp32 (see F32OUT): a handful of shapes of the kernel is enough, the path is not a hot one
+template <int QT, typename AT>
+static int launch_gemv_f32out(const void *x, const void *w, void *y, int layout, int M, int N, int K, hipStream_t st) {
+    const bool tiled_ok = layout == LAYOUT_TILED && (N % TILE_ROWS) == 0 && (K % TILE_COLS) == 0;
+    if (layout == LAYOUT_TILED && !tiled_ok) return -5;
+    if (tiled_ok) {
+        for (int m0 = 0; m0 < M; m0 += 16) {
+            const int mc = (M - m0) < 16 ? (M - m0) : 16;
+            const AT *xp = (const AT *)x + (int64_t)m0 * K;
+            AT *yp = (AT *)((float *)y + (int64_t)m0 * N);
+            const uint8_t *wp = (const uint8_t *)w;
+            if (mc <= 2) launch_mfma<QT, AT, 1, 2, 1, false, 0, 1, true>(xp, wp, yp, mc, N, K, 0, st);
+            else if (mc <= 4) launch_mfma<QT, AT, 1, 2, 2, false, 0, 1, true>(xp, wp, yp, mc, N, K, 0, st);
+            else if (mc <= 8) launch_mfma<QT, AT, 2, 1, 2, false, 0, 1, true>(xp, wp, yp, mc, N, K, 0, st);
+            else launch_mfma<QT, AT, 4, 2, 8, false, 0, 1, true>(xp, wp, yp, mc, N, K, 0, st);
+        }
+        return 0;
+    }
+    for (int m0 = 0; m0 < M; m0 += 4)
+        hipLaunchKernelGGL((gemv_generic_kernel<QT, LAYOUT_GGML, AT, 4, true>), dim3((N + 3) / 4), dim3(256), 0, st,
+                           (const AT *)x, (const uint8_t *)w, (AT *)y, m0, M, N, K);
+    return 0;
 }
 
 template <int QT, typename AT>
@@ -455,7 +497,7 @@ static int launch_gemv_t(const void *x, const void *w, void *y, int layout, int 
         return 0;
     }
     for (int m0 = 0; m0 < M; m0 += 4)
-        hipLaunchKernelGGL((gemv_generic_kernel<QT, LAYOUT_GGML, AT, 4>), dim3((N + 3) / 4), dim3(256), 0, st,
+        hipLaunchKernelGGL((gemv_generic_kernel<QT, LAYOUT_GGML, AT, 4, false>), dim3((N + 3) / 4), dim3(256), 0, st,
                            (const AT *)x, (const uint8_t *)w, (AT *)y, m0, M, N, K);
     return 0;
 }
@@ -534,6 +576,20 @@ int launch_moe_gemv(const void *x, const int32_t *ids, const float *route_w, int
     case QT_SYM_INT8: return launch_moe_q<QT_SYM_INT8>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, act_dtype, hidden, inter, act, st);
     case QT_NF4: return launch_moe_q<QT_NF4>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, act_dtype, hidden, inter, act, st);
     case QT_FP8_E4M3: return launch_moe_q<QT_FP8_E4M3>(x, ids, route_w, slots, n_exp, gates, ups, downs, h, y, act_dtype, hidden, inter, act, st);
+    default: return -2;
+    }
+}
+
+// x: bf16 [M, K]; y: float [M, N]
+int launch_gemv_bf16_f32out(const void *x, const void *w, void *y, int qtype, int layout, int M, int N, int K,
+                            hipStream_t st) {
+    if (M == 0 || N == 0) return 0;
+    switch (qtype) {
+    case QT_SYM_INT4: return launch_gemv_f32out<QT_SYM_INT4, __bf16>(x, w, y, layout, M, N, K, st);
+    case QT_ASYM_INT4: return launch_gemv_f32out<QT_ASYM_INT4, __bf16>(x, w, y, layout, M, N, K, st);
+    case QT_SYM_INT8: return launch_gemv_f32out<QT_SYM_INT8, __bf16>(x, w, y, layout, M, N, K, st);
+    case QT_NF4: return launch_gemv_f32out<QT_NF4, __bf16>(x, w, y, layout, M, N, K, st);
+    case QT_FP8_E4M3: return launch_gemv_f32out<QT_FP8_E4M3, __bf16>(x, w, y, layout, M, N, K, st);
     default: return -2;
     }
 }

@@ -208,6 +208,22 @@ def lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, work
                                  stream), "lowbit_gemm_ring")
 
 
+_lib.lowbit_forward_f32_workspace_bytes.argtypes = [c_int64, c_int64, c_int64]
+_lib.lowbit_forward_f32_workspace_bytes.restype = c_size_t
+_lib.lowbit_forward_f32.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int64, c_int64, c_void_p,
+                                    c_size_t, c_void_p]
+_lib.lowbit_forward_f32.restype = c_int
+
+
+def lowbit_forward_f32_workspace_bytes(m, n, k) -> int:
+    return _lib.lowbit_forward_f32_workspace_bytes(m, n, k)
+
+
+def lowbit_forward_f32(x, w, y, qtype, layout, m, n, k, workspace, workspace_bytes, stream):
+    _check(_lib.lowbit_forward_f32(x, w, y, qtype, layout, m, n, k, workspace, workspace_bytes, stream),
+           "lowbit_forward_f32")
+
+
 _lib.lowbit_noalloc_scratch_bytes.argtypes = []
 _lib.lowbit_noalloc_scratch_bytes.restype = c_size_t
 _lib.lowbit_forward_noalloc.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,

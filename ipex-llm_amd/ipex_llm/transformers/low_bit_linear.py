@@ -217,20 +217,34 @@ def _as_u8(w):
     return w.view(torch.uint8) if w.dtype != torch.uint8 else w
 
 
-def forward_new(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int, layout: int = None):
-    """xe_linear.forward_new: y[M, out] = x[M, K] @ dequant(w)[out, K]^T in x.dtype."""
+def forward_new(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int, layout: int = None,
+                keep_fp32: bool = False):
+    """xe_linear.forward_new: y[M, out] = x[M, K] @ dequant(w)[out, K]^T in x.dtype.
+
+    A float32 x is computed in half precision (what LowBitLinear asks for at M > 1, low_bit_linear.py:660-665
+    of the reference) unless keep_fp32 is set: then x and y stay fp32 through lowbit_forward_f32."""
     invalidInputError(x.dim() == 2 and x.device.type == _ACCEL and w.device == x.device,
                       "forward_new expects a 2-D activation and a weight on the same GPU")
     invalidInputError(x.dtype in _DT, f"unsupported activation dtype {x.dtype}")
     m, k = x.shape
     if layout is None:
         layout = device_layout(qtype, (output_size, k))
-    xc = x if x.dtype != torch.float32 else x.half()
-    xc = xc.contiguous()
     w = _as_u8(w)
     invalidInputError(w.numel() == ggml.lowbit_blob_bytes(qtype, output_size * k),
                       f"weight blob has {w.numel()} bytes, expected "
                       f"{ggml.lowbit_blob_bytes(qtype, output_size * k)} for [{output_size}, {k}]")
+    if keep_fp32 and x.dtype == torch.float32:
+        xc = x.contiguous()
+        y = torch.empty((m, output_size), dtype=torch.float32, device=x.device)
+        if m and output_size:
+            with torch.cuda.device(x.device):
+                ws_bytes = ggml.lowbit_forward_f32_workspace_bytes(m, output_size, k)
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+                ggml.lowbit_forward_f32(xc.data_ptr(), w.data_ptr(), y.data_ptr(), qtype, layout, m, output_size, k,
+                                        ws.data_ptr(), ws_bytes, _stream())
+        return y
+    xc = x if x.dtype != torch.float32 else x.half()
+    xc = xc.contiguous()
     y = torch.empty((m, output_size), dtype=xc.dtype, device=x.device)
     if m and output_size:
         with torch.cuda.device(x.device):
@@ -249,11 +263,12 @@ def forward_new(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int, 
 
 
 def batch_forward(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int = None, layout: int = None):
-    """xe_batch.batch_forward: same product, 1 < M <= 16 (one pass over the weights)."""
+    """xe_batch.batch_forward: same product, 1 < M <= 16 (one pass over the weights).  The reference hands it
+    x in the dtype it has (low_bit_linear.py:657-659), so a float32 x stays fp32."""
     if output_size is None:
         k = x.shape[1]
         output_size = _as_u8(w).numel() // ggml.ggml_type_size(qtype) * ggml.ggml_qk_size(qtype) // k
-    return forward_new(x, w, qtype, output_size, layout)
+    return forward_new(x, w, qtype, output_size, layout, keep_fp32=True)
 
 
 def dequant(x: torch.Tensor, w: torch.Tensor, qtype: int, layout: int = None, shape=None):
@@ -558,9 +573,11 @@ class LowBitLinear(nn.Linear):
                 if use_batch_forward(x_2d, self.weight.qtype, self.out_len):
                     result = batch_forward(x_2d, w, self.qtype, self.out_len, layout=layout)
                 else:
-                    # fp32 activations are computed in half precision, as the reference does
-                    # for M > 1 (low_bit_linear.py:660-665); forward_new casts back
-                    result = forward_new(x_2d, w, self.qtype, self.out_len, layout=layout)
+                    # A float32 x is computed in half precision only where the reference does so: at inference
+                    # with conver_to_half and more than one row (low_bit_linear.py:660-665).  One row, or a layer
+                    # built with conver_to_half=False, keeps fp32 in and out (:666-668).
+                    to_half = not is_training and self.conver_to_half and x_2d.shape[0] > 1
+                    result = forward_new(x_2d, w, self.qtype, self.out_len, layout=layout, keep_fp32=not to_half)
                 if do_empty_cache:
                     torch.cuda.empty_cache()
             result = result.view(new_shape)

@@ -280,3 +280,66 @@ def test_module_cuda_and_cpu_keep_the_residency_rule(qname):
     # quantize(device) lands tiled too
     direct = FP4Params(w.clone(), qtype=qtype).quantize("cuda")
     assert torch.equal(direct.data.view(torch.uint8), born.data.view(torch.uint8))
+
+
+# ------------------------------------------------------------------ fp32 activations
+
+@pytest.mark.parametrize("qname", ["sym_int4", "asym_int4", "sym_int8", "nf4", "fp8_e4m3"])
+@pytest.mark.parametrize("m,n,k", [(1, 96, 1024), (3, 272, 384), (20, 64, 512), (2, 37, 256)])
+def test_forward_f32_keeps_range_and_precision(qname, m, n, k):
+    """lowbit_forward_f32 (fp32 in, fp32 out): activations of magnitude 1e5 must neither overflow nor lose
+    more than the parity bar allows, and the result carries far more than half precision."""
+    from ipex_llm.transformers.low_bit_linear import forward_new
+    qtype = Q[qname]
+    if k % orc.qk_size(qtype):
+        pytest.skip("row length is no multiple of the block")
+    rng = np.random.default_rng(300 + m)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = (rng.standard_normal((m, k)) * 1e5).astype(np.float32)          # far beyond fp16's 65504
+    blob = orc.quantize(w, qtype)
+    p = FP4Params(torch.from_numpy(w), qtype=qtype).to("cuda")
+    y = forward_new(torch.from_numpy(x).cuda(), p.data, qtype, n, layout=p.blob_layout, keep_fp32=True)
+    assert y.dtype == torch.float32
+    y = y.cpu().numpy()
+    ref = orc.mul_mat_q(blob, x, (n, k), qtype)
+    exact = orc.mul_mat_exact(blob, x, (n, k), qtype)
+    assert np.isfinite(y).all()
+    assert np.abs(y - ref).max() <= 1e-2 * np.abs(ref).max()
+    assert np.abs(y - exact).max() <= 3e-5 * np.abs(exact).max()           # two bf16 planes: 16 mantissa bits
+
+
+def test_lowbitlinear_float32_input_follows_the_reference_rules():
+    """low_bit_linear.py:657-668 of the reference: float32 x goes to half precision only at inference with
+    conver_to_half and more than one row outside the small-batch range."""
+    torch.manual_seed(8)
+    w = torch.randn(64, 256) * 0.02
+    blob = orc.quantize(w.numpy(), Q["sym_int4"])
+
+    def layer(conver_to_half):
+        lin = LowBitLinear(256, 64, Q["sym_int4"], bias=False, conver_to_half=conver_to_half).eval()
+        lin.weight = FP4Params(w.clone(), qtype=Q["sym_int4"])
+        return lin.to("cuda")
+    big = 3.0e5                                                            # overflows fp16
+    for rows, conv, stays_fp32 in ((1, True, True), (4, True, True), (40, True, False), (40, False, True)):
+        x = torch.randn(rows, 256) * (big if stays_fp32 else 1.0)
+        y = layer(conv)(x.cuda())
+        assert y.dtype == torch.float32 and torch.isfinite(y).all()
+        exact = orc.mul_mat_exact(blob, x.numpy(), (64, 256), Q["sym_int4"])
+        tol = 3e-5 if stays_fp32 else 2e-3
+        assert np.abs(y.cpu().numpy() - exact).max() <= tol * np.abs(exact).max(), (rows, conv)
+
+
+def test_cpu_resident_matmul_is_fp32_in_and_out():
+    """ggml_compute_forward_mul_mat_q_fp32 (the reference's CPU branch, low_bit_linear.py:462-497): |x| up to
+    1e5 and |y| far above 65504 stay finite and within the parity bar of the reference-style CPU matmul."""
+    from ipex_llm.transformers.low_bit_linear import ggml_matmul_src1_x_src0_t
+    rng = np.random.default_rng(9)
+    for qname in ("sym_int4", "asym_int4", "sym_int8"):
+        qtype = Q[qname]
+        w = (rng.standard_normal((48, 512)) * 0.5).astype(np.float32)
+        x = (rng.standard_normal((5, 512)) * 1e5).astype(np.float32)
+        blob = orc.quantize(w, qtype)
+        y = ggml_matmul_src1_x_src0_t(torch.from_numpy(blob), torch.from_numpy(x), torch.Size((48, 512)), qtype).numpy()
+        ref = orc.mul_mat_q(blob, x, (48, 512), qtype)
+        assert np.isfinite(y).all() and np.abs(ref).max() > 65504
+        assert np.abs(y - ref).max() <= 1e-2 * np.abs(ref).max()
