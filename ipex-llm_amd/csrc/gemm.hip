@@ -21,27 +21,35 @@ namespace lowbit {
 int launch_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 int waves, hipStream_t st);
 
-constexpr int GM = 128;          // rows of x per workgroup
+constexpr int GM = 128;          // rows of x per workgroup (the tall form below takes 256)
 constexpr int GN_WAVE = 64;      // weight rows per wave
 constexpr int GN = 256;          // weight rows per workgroup (4 waves)
 
 constexpr int MB32 = GM / 32;        // 32-row blocks of x per workgroup
 constexpr int NB32 = GN_WAVE / 32;   // 32-row blocks of W per wave (two tiles each)
+constexpr int GM_TALL = 256, MB32_TALL = GM_TALL / 32;
 
 // Operand layout of v_mfma_f32_32x32x16: lane l = 32*kg + i holds 8 consecutive k (8*kg .. +7 of
 // the 16-column step) of row/column i.  A 32-row weight block is two tiles (rows 0-15, 16-31);
 // in a tile, lane slot 16*c + r holds columns 8*c .. +7 of each 32-column sub-block, so lane
 // (kg, i) takes slot 16*kg + i%16 of tile i/16 for the first 16 columns of every sub-block
 // ("lo" registers) and slot 16*(kg+2) + i%16 for the second 16 columns ("hi" registers).
-template <int QT, typename AT, bool DMA>
-__global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+//
+// MB = 32-row blocks of x per workgroup: 4 (128 rows) or, for the tall form, 8 (256 rows, DMA form only).  The
+// tall form dequantizes every weight once per 256 rows of x: half the VALU work, half the weight loads and
+// half the barriers per MFMA; its 16 accumulator blocks take all 256 accumulation registers, so a CU holds
+// one workgroup.  tn0 / tn_cnt: the launch covers the column tiles tn0 .. tn0 + tn_cnt - 1 of y.
+template <int QT, typename AT, bool DMA, int MB>
+__global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                         AT *__restrict__ y, int M, int N, int K, int xcd_m,
                                                         const int32_t *__restrict__ group_offsets,
                                                         const uint8_t *const *__restrict__ group_weights,
                                                         int n_groups, int max_mtiles, int k_steps,
-                                                        float *__restrict__ ws) {
+                                                        float *__restrict__ ws, int tn0, int tn_cnt) {
     using F = Fmt<QT>;
     using V8 = typename Vec8<AT>::type;
+    static_assert(MB == 4 || (MB == 8 && DMA), "row tiles of 128 rows, or 256 rows in the DMA form");
+    constexpr int MB32 = MB, GM = 32 * MB;            // shadow the 128-row constants of the file
     // x block of a K step: 8 * MB32 pieces of 1 KiB (layout below), double buffered
     __shared__ __attribute__((aligned(16))) uint8_t xs0[8 * MB32 * 1024];
     __shared__ __attribute__((aligned(16))) uint8_t xs1[8 * MB32 * 1024];
@@ -50,7 +58,8 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODEBOOK[threadIdx.x];
     }
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: scalar address arithmetic
     const int G = K / TILE_COLS;
     const int n_tiles = N / TILE_ROWS;
 
@@ -60,7 +69,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
     // column-tile) and sees each weight tile from all its row-tiles at about the same time.
     int m0, tile_n;
     if (group_offsets == nullptr) {
-        const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
+        const int tiles_m = (M + GM - 1) / GM, tiles_n = tn_cnt;
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
         const int band_m = (tiles_m + xcd_m - 1) / xcd_m;
         const int xcd_n = 8 / xcd_m;
@@ -68,6 +77,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         const int tile_m = (xcd % xcd_m) * band_m + slot % band_m;
         tile_n = (xcd / xcd_m) * band_n + slot / band_m;
         if (slot >= band_m * band_n || tile_m >= tiles_m || tile_n >= tiles_n) return;   // whole workgroup leaves
+        tile_n += tn0;
         m0 = tile_m * GM;
     } else {
         // Grouped mode (mixture-of-experts): rows group_offsets[e] .. group_offsets[e+1]-1 of x use
@@ -129,9 +139,10 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             xl[i] = (((chunk >> 3) * (4 * MB32) + (row_in >> 3)) * 64 + (chunk & 7) * 8 + (row_in & 7)) * 16;
         }
     } else {
-        xrow0 = m0 + 64 * (wave & 1) + (lane & 7);
+        xrow0 = m0 + (GM / 2) * (wave & 1) + (lane & 7);
         xcol = (wave >> 1) * 128 + (lane >> 3) * 16;
     }
+    constexpr int PW = 2 * MB32;                     // pieces of 1 KiB (8 rows of a half row) a wave fetches per K step
     // Split-K: with a workspace the grid has a second dimension, workgroup (t, s) walks the K steps
     // s * k_steps .. and leaves its fp32 partial tile in ws[s]; a second kernel sums the splits.  It
     // fills the machine when the output alone has too few tiles (small M, narrow N).
@@ -148,16 +159,32 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         // explicit vmcnt(0) ahead of the workgroup barrier that publishes the buffer.
         const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
         const uint32_t lbase = __builtin_amdgcn_readfirstlane(
-            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + wave * 8 * 1024);
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + wave * PW * 1024);
         uint32_t row = xrow0 + 8 * j;
         row = row < (uint32_t)M ? row : (uint32_t)M - 1;
         const uint8_t *src = xk + (__umul24(row, (uint32_t)K * (uint32_t)sizeof(AT)) + xcol);
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                      :: "v"(src), "s"(lbase + j * 1024) : "memory", "m0");
     };
+    // Tall form (whole 256-row tiles only, so no row is clamped): the per-lane part of the address is a
+    // constant 32-bit offset and everything that changes from load to load is scalar arithmetic.
+    const uint32_t xlane_off = (uint32_t)(lane & 7) * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)(lane >> 3) * 16u;
+    const uint64_t xwave_base = (uint64_t)(uintptr_t)x +
+        ((uint64_t)(m0 + (GM / 2) * (wave & 1)) * (uint64_t)K + (uint64_t)(wave >> 1) * 64u) * sizeof(AT);
+    auto dma_x_scalar = [&](int kt, uint8_t *buf, int j) {
+        kt = kt0 + (kt < last ? kt : last);
+        const uint64_t src = xwave_base + (uint64_t)kt * (TILE_COLS * sizeof(AT)) + (uint64_t)j * 8u * (uint64_t)K * sizeof(AT);
+        const uint32_t lbase = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + (wave * PW + j) * 1024);
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(xlane_off), "s"(src), "s"(lbase) : "memory", "m0");
+    };
     auto dma_x = [&](int kt, uint8_t *buf) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) dma_x_one(kt, buf, j);
+        for (int j = 0; j < PW; j++) {
+            if constexpr (MB32 == 8) dma_x_scalar(kt, buf, j);
+            else dma_x_one(kt, buf, j);
+        }
     };
     auto load_x = [&](int kt, u32x4 (&xr)[8]) {
         kt = kt0 + (kt < last ? kt : last);              // past the end: a harmless re-read, never used
@@ -195,16 +222,21 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         if constexpr (F::BITS == 8) t.hi[nb].q1 = ld<u32x4>(tile + 1024 + slot_hi * 16);
     };
 
-    // what goes out after 16-column step ks: everything within the first five of the eight steps, so
-    // that the data has the rest of the K step to arrive (later placements end in a longer wait at
-    // the barrier, a single burst at ks = 0 stalls the waves at the address unit)
-    auto fetch_part = [&](int kt, uint8_t *buf, WRegs &t, int ks) {
-        if (ks < 2) {
-            load_w_nb(kt, t, ks);
-            dma_x_one(kt, buf, ks);
-        } else if (ks < 5) {
-            dma_x_one(kt, buf, 2 * ks - 2);
-            dma_x_one(kt, buf, 2 * ks - 1);
+    // The loads of the next K step, as NB32 + PW units (the weight registers of a 32-row block; one piece of x),
+    // dealt out over the first five eighths of the step's MFMA groups, so that the data has the rest of the
+    // step to arrive and no group carries more than a load or two: a burst stalls the waves at the CU's
+    // address unit (41 % of a K step at M = 2048 when all loads of a step went out together), and with one or
+    // two waves per SIMD every cycle a wave stands at a memory instruction is a cycle its MFMA pipe idles.
+    // `point` = index of the MFMA group (16-column step * row blocks + row block) the call follows.
+    auto fetch_units = [&](int kt, uint8_t *buf, WRegs &t, const int point, const int points) {
+        constexpr int UNITS = NB32 + PW;
+        const int spread = points * 5 / 8 > 0 ? points * 5 / 8 : 1;
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            if (u < point * UNITS / spread || u >= (point + 1) * UNITS / spread || point >= spread) continue;
+            if (u < NB32) load_w_nb(kt, t, u);
+            else if constexpr (MB32 == 8) dma_x_scalar(kt, buf, u - NB32);
+            else dma_x_one(kt, buf, u - NB32);
         }
     };
 
@@ -236,7 +268,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
     const int xlane = (i32 >> 3) * 1024 + kg * 128 + (i32 & 7) * 16;
     auto compute = [&](const uint8_t *cur, const WRegs &t, auto mbc_, auto &&between) {
         constexpr int MBC = decltype(mbc_)::value;
-        constexpr int PER = (4 * NB32) / (MBC * NB32);        // dequantized pairs per MFMA slot
+        constexpr int SLOTS = MBC * NB32, PAIRS = 4 * NB32;   // MFMAs per 16-column step; register pairs to dequantize meanwhile
         V8 xv[MBC];
         u32x4 wv[NB32];
 #pragma unroll
@@ -254,10 +286,12 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
                 for (int nb = 0; nb < NB32; nb++) {
                     mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
                     if (ks < 7) {
+                        // pairs [slot * PAIRS / SLOTS, (slot + 1) * PAIRS / SLOTS): spread evenly over the MFMA slots
+                        const int slot_i = mb * NB32 + nb;
 #pragma unroll
-                        for (int q = 0; q < PER; q++) {
-                            const int idx = (mb * NB32 + nb) * PER + q;   // 0 .. 4*NB32-1: (weight block, pair)
-                            wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);
+                        for (int idx = 0; idx < PAIRS; idx++) {
+                            if (idx < slot_i * PAIRS / SLOTS || idx >= (slot_i + 1) * PAIRS / SLOTS) continue;
+                            wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);   // (weight block, pair)
                         }
                     }
                 }
@@ -265,9 +299,9 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
                 // keep this order: the scheduler does not know how long an MFMA takes and would
                 // sink the LDS read down to its first use, exposing the LDS latency every time
                 __builtin_amdgcn_sched_barrier(0);
+                between(ks * MBC + mb, 8 * MBC);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            between(ks);
-            __builtin_amdgcn_sched_barrier(0);
             if (ks < 7) {
 #pragma unroll
                 for (int nb = 0; nb < NB32; nb++) wv[nb] = wn[nb];
@@ -275,7 +309,7 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         }
     };
     typedef std::integral_constant<int, MB32> full_t;
-    auto nothing = [](int) {};
+    auto nothing = [](int, int) {};
 
     auto epilogue = [&](auto mbc_) {
         constexpr int MBC = decltype(mbc_)::value;
@@ -338,13 +372,13 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
             wait_all_loads();
             __syncthreads();
             for (int kt = 0; kt + 1 < Gs; kt += 2) {
-                compute(xs0, w0, mbc, [&](int ks) {
-                    fetch_part(kt + 1, xs1, w1, ks);
+                compute(xs0, w0, mbc, [&](const int point, const int points) {
+                    fetch_units(kt + 1, xs1, w1, point, points);
                 });
                 wait_all_loads();
                 __syncthreads();
-                compute(xs1, w1, mbc, [&](int ks) {          // past the end: clamped, unused re-reads
-                    fetch_part(kt + 2, xs0, w0, ks);
+                compute(xs1, w1, mbc, [&](const int point, const int points) {   // past the end: clamped, unused re-reads
+                    fetch_units(kt + 2, xs0, w0, point, points);
                 });
                 wait_all_loads();
                 __syncthreads();
@@ -353,7 +387,11 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
         };
         // tail tiles and small expert groups: 32-row blocks without rows of x skip their MFMAs
         const int mb_cnt = (M - m0 + 31) / 32;
-        if (mb_cnt <= 1) {
+        if constexpr (MB32 == 8) {
+            // the launcher hands the tall form whole 256-row tiles only
+            run(full_t());
+            epilogue(full_t());
+        } else if (mb_cnt <= 1) {
             run(std::integral_constant<int, 1>());
             epilogue(std::integral_constant<int, 1>());
         } else if (mb_cnt <= 2) {
@@ -379,9 +417,12 @@ __global__ __launch_bounds__(256, DMA ? 2 : 1) void gemm_mfma_kernel(const AT *_
 
 #define LOWBIT_GEMM_STEP(i, cur, nxt, xst, xld, wc, wl)                        \
     if (kt + (i) < Gs) {                                                       \
-        compute(cur, wc, full_t(), [&](int ks) {                               \
-            if (ks < 2) load_w_nb(kt + (i) + 2, wl, ks);                       \
-            load_x_one(kt + (i) + 2, xld, ks);                                 \
+        compute(cur, wc, full_t(), [&](const int point, const int points) {    \
+            if (point % MB32 == MB32 - 1) {                                    \
+                const int ks = point / MB32;                                   \
+                if (ks < 2) load_w_nb(kt + (i) + 2, wl, ks);                   \
+                load_x_one(kt + (i) + 2, xld, ks);                             \
+            }                                                                  \
         });                                                                    \
         store_x(nxt, xst);                                                     \
         __syncthreads();                                                       \
@@ -468,16 +509,56 @@ int gemm_splits(int M, int N, int K, size_t ws_bytes) {
     return best;
 }
 
+// How many column tiles (256 weight rows each) the tall form takes, from the left: whole rounds of one
+// 256 x 256 tile per CU, so that no CU sits idle while another still works on a second tall tile; the 128-row
+// form covers the columns that are left.  0 = the tall form is not used: M not a multiple of 256, too few
+// tiles to fill the machine once, K too long for 24-bit row offsets - or columns left over that would not
+// fill the machine themselves.  Measured on MI355X: a machine full of tall tiles runs 4-7 % (sym_int4) to
+// 10 % (nf4) faster than the 128-row form with two workgroups per CU, which the idle CUs of a thin remainder
+// eat up again ([11008 x 4096] at M = 2048: 32 tall columns + 11 left over, no faster than 688 small tiles).
+static int tall_columns(int M, int N, int K, int n_cus) {
+    if (M < 2 * GM_TALL || M % GM_TALL || M >= (1 << 24) || K >= (1 << 23)) return 0;
+    const int tiles_m = M / GM_TALL, tiles_n = (N + GN - 1) / GN;
+    const int rounds = tiles_m * tiles_n / n_cus;
+    if (rounds < 1) return 0;
+    int cols = rounds * n_cus / tiles_m;
+    if (cols >= tiles_n) return tiles_n;
+    const int left = (tiles_n - cols) * (M / GM);        // 128-row tiles of the remainder
+    return 2 * left >= 3 * n_cus ? cols : 0;
+}
+
 template <int QT, typename AT>
 static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, int K, float *ws, int splits,
                          hipStream_t st) {
-    const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
+    if (splits <= 1) ws = nullptr;
+    const int G = K / TILE_COLS;
+    const int tiles_n_all = (N + GN - 1) / GN;
+    static const int n_cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            n = 256;
+        return n > 0 ? n : 256;
+    }();
+    // tall form on the left columns, 128-row form on the rest (both in the same stream, the second starts when
+    // the tall tiles, which all take the same time, are done)
+    const int tall = ws ? 0 : tall_columns(M, N, K, n_cus);
+    if (tall > 0) {
+        const int tiles_m = M / GM_TALL;
+        int xcd_m = 1;
+        while (xcd_m * 2 <= 8 && xcd_m * 2 <= tiles_m) xcd_m *= 2;
+        const int xcd_n = 8 / xcd_m;
+        const int band_m = (tiles_m + xcd_m - 1) / xcd_m, band_n = (tall + xcd_n - 1) / xcd_n;
+        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL>), dim3(8 * band_m * band_n), dim3(256), 0, st,
+                           (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr,
+                           (const uint8_t *const *)nullptr, 0, 0, G, (float *)nullptr, 0, tall);
+        if (tall == tiles_n_all) return 0;
+    }
+    const int tn0 = tall, tiles_n = tiles_n_all - tall;
+    const int tiles_m = (M + GM - 1) / GM;
     int xcd_m = 1;                                       // XCDs along M: power of two <= min(8, tiles_m)
     while (xcd_m * 2 <= 8 && xcd_m * 2 <= tiles_m) xcd_m *= 2;
     const int xcd_n = 8 / xcd_m;
     const int band_m = (tiles_m + xcd_m - 1) / xcd_m, band_n = (tiles_n + xcd_n - 1) / xcd_n;
-    if (splits <= 1) ws = nullptr;
-    const int G = K / TILE_COLS;
     const int k_steps = ws ? (G + splits - 1) / splits : G;
     const int ny = ws ? (G + k_steps - 1) / k_steps : 1;             // splits that actually hold steps
     dim3 grid(8 * band_m * band_n, ny);
@@ -487,13 +568,13 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     // form with its deeper prefetch is faster.
     const bool dma = tiles_m * tiles_n * ny > 256 && M < (1 << 24) && K < (1 << 23);   // 24-bit row offsets
     if (dma)
-        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
+        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
                            (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0,
-                           k_steps, ws);
+                           k_steps, ws, tn0, tiles_n);
     else
-        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, false>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
+        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, false, MB32>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
                            (AT *)y, M, N, K, xcd_m, (const int32_t *)nullptr, (const uint8_t *const *)nullptr, 0, 0,
-                           k_steps, ws);
+                           k_steps, ws, tn0, tiles_n);
     if (ws) {
         const int64_t threads = (int64_t)tiles_m * tiles_n * (GM * GN / 4);
         hipLaunchKernelGGL((splitk_reduce_kernel<AT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, ws,
@@ -507,9 +588,9 @@ static int launch_grouped_t(const void *x, const void *const *w, void *y, const 
                             int total_rows, int N, int K, hipStream_t st) {
     const int max_mtiles = (total_rows + GM - 1) / GM + n_groups;    // every group adds at most one partial tile
     const int tiles_n = (N + GN - 1) / GN;
-    hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true>), dim3(tiles_n * max_mtiles), dim3(256), 0, st, (const AT *)x,
+    hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32>), dim3(tiles_n * max_mtiles), dim3(256), 0, st, (const AT *)x,
                        (const uint8_t *)nullptr, (AT *)y, 0, N, K, 1, offsets, (const uint8_t *const *)w, n_groups,
-                       max_mtiles, 0, (float *)nullptr);
+                       max_mtiles, 0, (float *)nullptr, 0, tiles_n);
     return 0;
 }
 

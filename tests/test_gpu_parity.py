@@ -335,3 +335,23 @@ def test_workspace_query_is_consistent():
         assert b % (32 * 256 * 4) == 0                              # whole partial tiles of either kernel
     assert ggml.lowbit_workspace_bytes(256, 4096, 11008) > 0        # 32 tiles, 86 steps: worth splitting
     assert ggml.lowbit_workspace_bytes(2048, 11008, 4096) == 0      # 688 tiles fill the machine
+
+
+@pytest.mark.parametrize("qtype,dtype", [(Q4_0, torch.float16), (Q4_1, torch.float16), (Q8_0, torch.bfloat16),
+                                         (NF4, torch.bfloat16), (FP8, torch.bfloat16)])
+@pytest.mark.parametrize("m,n,k", [(1024, 16384, 256), (512, 33024, 384), (768, 22016, 128)])
+def test_gemm_tall_row_tiles_against_oracle(qtype, dtype, m, n, k):
+    """Shapes whose 256 x 256 tiles fill every CU at least once take the form of the GEMM with 256-row tiles on
+    the left columns and the 128-row form on the columns left over (one column tile of 33024 = 129 * 256, 22
+    of 22016 = 86 * 256 at three row tiles); K of one, two and three 128-column steps.  Oracle on sampled rows
+    of W and x."""
+    w = weights(5600 + qtype + m, (n, k), outliers=False)
+    x = acts(5601 + m, m, k, dtype)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n, fn="gemm")
+    assert np.isfinite(y).all()
+    rows = np.unique(np.concatenate([np.arange(0, n, 61), np.arange(n - 300, n)]))      # incl. the last column tiles
+    ms = np.unique(np.concatenate([np.arange(0, m, 37), [255, 256, m - 1]]))
+    y_exact = orc.mul_mat_exact(orc.quantize(w[rows], qtype), x.float().numpy()[ms], (len(rows), k), qtype)
+    tol = 2e-3 if dtype == torch.float16 else 8e-3
+    assert np.abs(y[np.ix_(ms, rows)] - y_exact).max() <= tol * np.abs(y_exact).max()
