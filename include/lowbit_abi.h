@@ -67,6 +67,10 @@ extern "C" {
 
 int lowbit_abi_version(void);
 const char *lowbit_last_error(void);
+/* What the HIP runtime reports for the current device: marketing and architecture name, number of CUs, maximum
+ * shader and memory clocks (kHz), memory bus width (bits).  For benchmark reports; any pointer may be null. */
+int lowbit_device_info(char *name, size_t name_bytes, int *compute_units, int *shader_clock_khz, int *memory_clock_khz,
+                       int *memory_bus_bits);
 
 /* ------------------------------------------------------------------ (1) */
 
@@ -176,6 +180,15 @@ int lowbit_dequantize(const void *w, void *dst, int qtype, int64_t N, int64_t K,
  * estimates to be faster for the shape. */
 int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
                    int64_t N, int64_t K, void *stream);
+/* Which kernel lowbit_forward (have_workspace = 0) or lowbit_forward_ws (a non-null workspace of
+ * workspace_bytes) runs for a shape with an 8-byte aligned y, without running anything: the streaming GEMV in 16-row passes, the ring kernel for batch
+ * sizes, or the MFMA GEMM with or without a K split.  Negative for an unknown qtype.  Host arithmetic only. */
+#define LOWBIT_PLAN_GEMV 0
+#define LOWBIT_PLAN_RING 1
+#define LOWBIT_PLAN_GEMM 2
+#define LOWBIT_PLAN_GEMM_SPLIT 3
+int lowbit_forward_plan(int qtype, int layout, int64_t M, int64_t N, int64_t K, int have_workspace,
+                        size_t workspace_bytes);
 /* The two kernels behind lowbit_forward, for callers (and benchmarks) that choose themselves.
  * waves = 0 lets the library pick the workgroup size of the GEMV. */
 int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,

@@ -81,6 +81,22 @@ static int check_weight_shape(const char *what, int qtype, int64_t N, int64_t K,
 extern "C" {
 
 int lowbit_abi_version(void) { return LOWBIT_ABI_VERSION; }
+
+int lowbit_device_info(char *name, size_t name_bytes, int *compute_units, int *shader_clock_khz, int *memory_clock_khz,
+                       int *memory_bus_bits) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (int rc = check_hip(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties")) return rc;
+    if (name && name_bytes) {
+        snprintf(name, name_bytes, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (shader_clock_khz) *shader_clock_khz = prop.clockRate;
+    if (memory_clock_khz) *memory_clock_khz = prop.memoryClockRate;
+    if (memory_bus_bits) *memory_bus_bits = prop.memoryBusWidth;
+    return 0;
+}
 const char *lowbit_last_error(void) { return g_err; }
 
 size_t ggml_type_size(int qtype) { return (size_t)type_size(qtype); }
@@ -220,17 +236,20 @@ size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 // 61 us however few rows it holds, where a GEMV pass takes 12 us.  With a workspace the GEMM can split
 // K over more workgroups at the price of writing and re-reading fp32 partial sums, and the ring kernel
 // (32 / 64 / 128-row tiles, units dealt out evenly) covers the batch sizes in between.
-static int forward_any(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
-                       int64_t N, int64_t K, void *workspace, size_t workspace_bytes, void *stream) {
-    if (M <= 16 || layout != LOWBIT_LAYOUT_TILED)
-        return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
-    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || K < 128)
-        return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);     // reports the error
+enum { PLAN_GEMV = LOWBIT_PLAN_GEMV, PLAN_RING = LOWBIT_PLAN_RING, PLAN_GEMM = LOWBIT_PLAN_GEMM,
+       PLAN_GEMM_SPLIT = LOWBIT_PLAN_GEMM_SPLIT };
+
+// which kernel, and for PLAN_GEMM_SPLIT into how many K splits
+static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, bool have_ws, size_t workspace_bytes,
+                        bool y_aligned8, int *splits_out) {
+    if (splits_out) *splits_out = 1;
+    if (M <= 16 || layout != LOWBIT_LAYOUT_TILED) return PLAN_GEMV;
+    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || K < 128) return PLAN_GEMM;     // reports the error
     const double passes = (double)((M + 15) / 16);
     // a pass cannot be shorter than its workgroups' walk along K (narrow weights leave CUs idle)
     const double stream_us = (double)lowbit_blob_bytes(qtype, N * K) / 2.8e6, walk_us = 0.07 * (double)(K / 128);
     const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
-    const int splits = workspace ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
+    const int splits = have_ws ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
     const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits);
     // The ring kernel (y 8-byte aligned) needs the workspace for its partial tiles; given that, it measured
     // faster than or level with the tiled GEMM, split or not, below M = 512 and about 7e10 FLOP (sym_int4 and
@@ -238,16 +257,33 @@ static int forward_any(const void *x, const void *w, void *y, int qtype, int lay
     // on the GEMM's tighter loop, it stays ahead at larger M as well while the GEMM's tiles are no more
     // than one per CU (Llama-3-70B set at M = 512 / 1024: 755 / 808 against 706 / 761 TFLOP/s).  Its own
     // estimate decides against the GEMV.
-    if (!(((uintptr_t)y) & 7) && workspace && ring_range(qtype, M, N, K) &&
-        ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes) {
-        if (ring_time_us((int)M, (int)N, (int)K, qtype, true) < t_gemv)
-            return lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, 0, stream);
-        return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
+    if (y_aligned8 && have_ws && ring_range(qtype, M, N, K) &&
+        ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes)
+        return ring_time_us((int)M, (int)N, (int)K, qtype, true) < t_gemv ? PLAN_RING : PLAN_GEMV;
+    if (t_gemv < t_gemm) return PLAN_GEMV;
+    if (splits > 1) {
+        if (splits_out) *splits_out = splits;
+        return PLAN_GEMM_SPLIT;
     }
-    if (t_gemv < t_gemm) return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
-    if (splits > 1)
+    return PLAN_GEMM;
+}
+
+extern "C" int lowbit_forward_plan(int qtype, int layout, int64_t M, int64_t N, int64_t K, int have_workspace,
+                                   size_t workspace_bytes) {
+    if (!qk_size(qtype) || M < 0 || N < 0 || K < 0) return -1;
+    return plan_forward(qtype, layout, M, N, K, have_workspace != 0, have_workspace ? workspace_bytes : 0, true, nullptr);
+}
+
+static int forward_any(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                       int64_t N, int64_t K, void *workspace, size_t workspace_bytes, void *stream) {
+    int splits = 1;
+    switch (plan_forward(qtype, layout, M, N, K, workspace != nullptr, workspace_bytes, !(((uintptr_t)y) & 7), &splits)) {
+    case PLAN_GEMV: return lowbit_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, stream);
+    case PLAN_RING: return lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, 0, stream);
+    case PLAN_GEMM_SPLIT:
         return lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, M, N, K, workspace, workspace_bytes, splits, stream);
-    return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);
+    default: return lowbit_gemm(x, w, y, qtype, layout, act_dtype, M, N, K, stream);
+    }
 }
 
 int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M, int64_t N,

@@ -50,6 +50,22 @@ _lib.lowbit_last_error.argtypes = []
 _lib.lowbit_last_error.restype = ctypes.c_char_p
 
 
+_lib.lowbit_device_info.argtypes = [ctypes.c_char_p, c_size_t, ctypes.POINTER(c_int), ctypes.POINTER(c_int),
+                                    ctypes.POINTER(c_int), ctypes.POINTER(c_int)]
+_lib.lowbit_device_info.restype = c_int
+
+
+def lowbit_device_info() -> dict:
+    """Name, CU count, maximum clocks and bus width of the current device as the HIP runtime reports them."""
+    name = ctypes.create_string_buffer(256)
+    cus, sclk, mclk, bus = c_int(), c_int(), c_int(), c_int()
+    _check(_lib.lowbit_device_info(name, 256, ctypes.byref(cus), ctypes.byref(sclk), ctypes.byref(mclk),
+                                   ctypes.byref(bus)), "lowbit_device_info")
+    return {"name": name.value.decode("utf-8", "replace"), "compute_units": cus.value,
+            "max_shader_clock_mhz": sclk.value / 1e3, "max_memory_clock_mhz": mclk.value / 1e3,
+            "memory_bus_bits": bus.value}
+
+
 def last_error() -> str:
     return (_lib.lowbit_last_error() or b"").decode("utf-8", "replace")
 
@@ -187,6 +203,16 @@ _lib.lowbit_gemm_ws.restype = c_int
 _lib.lowbit_gemm_ring.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64,
                                   c_void_p, c_size_t, c_int, c_void_p]
 _lib.lowbit_gemm_ring.restype = c_int
+
+
+_lib.lowbit_forward_plan.argtypes = [c_int, c_int, c_int64, c_int64, c_int64, c_int, c_size_t]
+_lib.lowbit_forward_plan.restype = c_int
+PLAN_GEMV, PLAN_RING, PLAN_GEMM, PLAN_GEMM_SPLIT = 0, 1, 2, 3
+
+
+def lowbit_forward_plan(qtype, layout, m, n, k, have_workspace, workspace_bytes=0) -> int:
+    """PLAN_* code of the kernel lowbit_forward (have_workspace False) / lowbit_forward_ws would run."""
+    return _lib.lowbit_forward_plan(qtype, layout, m, n, k, int(bool(have_workspace)), workspace_bytes)
 
 
 def lowbit_workspace_bytes(m, n, k) -> int:

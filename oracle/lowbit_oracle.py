@@ -30,6 +30,21 @@ def build(force=False):
 _lib = None
 
 
+def use_fast_build():
+    """Switches to the -O3 AVX2 build of the same source (for timing only: bench.py's cpu_baseline).  Has to be
+    called before the first use; returns the ISA string of the build that will be loaded."""
+    global _SO
+    fast = os.path.join(_HERE, "liblowbit_oracle_avx2.so")
+    try:
+        flags = open("/proc/cpuinfo").read().split("flags", 1)[1].split("\n", 1)[0].split()
+    except Exception:  # noqa: BLE001
+        flags = []
+    if _lib is None and os.path.exists(fast) and all(f in flags for f in ("avx2", "fma", "f16c")):
+        _SO = fast
+        return "gcc -O3 -mavx2 -mfma -mf16c (auto-vectorized C)"
+    return "gcc -O2 (portable x86-64 C)"
+
+
 def lib():
     global _lib
     if _lib is None:

@@ -297,3 +297,38 @@ def test_fused_mlp_refuses_weights_that_are_not_tiled_blobs_next_to_x():
     got = m(xf)                                                           # dense CPU weights: cannot be fused
     assert torch.equal(got, want) and m.calls == 2                        # the class's own forward ran
     assert fuse_mlp_base(m, 0, xf).shape == (2, 128)
+
+
+def test_kernel_choice_boundaries_are_pinned():
+    """Which kernel lowbit_forward / lowbit_forward_ws picks is decided by constants fitted on MI355X
+    (abi.hip, gemm.hip, gemm_ring.hip).  This table pins today's choices for the BASELINE shapes so that a
+    re-fit cannot silently route a shape to another kernel: whoever changes a constant re-measures and edits
+    the table.  Host arithmetic only (lowbit_forward_plan)."""
+    G, R, M, S = ggml.PLAN_GEMV, ggml.PLAN_RING, ggml.PLAN_GEMM, ggml.PLAN_GEMM_SPLIT
+
+    def plans(qtype, n, k, ms):
+        with_ws = [ggml.lowbit_forward_plan(qtype, 1, m, n, k, True, ggml.lowbit_workspace_bytes(m, n, k)) for m in ms]
+        without = [ggml.lowbit_forward_plan(qtype, 1, m, n, k, False) for m in ms]
+        return with_ws, without
+    ms = (1, 16, 17, 32, 64, 128, 256, 511, 512, 1024, 2048)
+    #                         1  16  17  32  64 128 256 511 512 1024 2048
+    table = {
+        (2, 4096, 4096):   ([G, G, G, G, R, R, R, R, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
+        (2, 11008, 4096):  ([G, G, R, R, R, R, R, R, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
+        (2, 4096, 11008):  ([G, G, R, R, R, R, R, R, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
+        (3, 11008, 4096):  ([G, G, R, R, R, R, R, R, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
+        (10, 8192, 8192):  ([G, G, R, R, R, R, R, R, R, R, M], [G, G, G, G, G, G, M, M, M, M, M]),
+        (10, 1024, 8192):  ([G, G, G, G, R, R, R, R, R, R, R], [G, G, G, G, G, G, G, M, M, M, M]),
+        (10, 28672, 8192): ([G, G, R, R, R, R, R, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
+        (10, 8192, 28672): ([G, G, R, R, R, R, R, R, R, R, M], [G, G, G, G, G, G, M, M, M, M, M]),
+        (8, 28672, 8192):  ([G, G, R, R, R, R, M, M, M, M, M], [G, G, M, M, M, M, M, M, M, M, M]),
+        (8, 8192, 28672):  ([G, G, R, R, R, R, S, S, S, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
+        (15, 14336, 4096): ([G, G, R, R, R, R, R, R, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
+    }
+    for (qtype, n, k), want in table.items():
+        assert plans(qtype, n, k, ms) == (want[0], want[1]), (qtype, n, k, plans(qtype, n, k, ms))
+    # the rules that do not depend on fitted constants
+    for qtype in (2, 3, 8, 10, 15):
+        assert ggml.lowbit_forward_plan(qtype, 1, 16, 4096, 4096, True, 1 << 30) == G        # one streaming pass
+        assert ggml.lowbit_forward_plan(qtype, 0, 4096, 4096, 4096, True, 1 << 30) == G      # ggml layout: any-shape kernel
+    assert ggml.lowbit_forward_plan(99, 1, 1, 64, 128, False) < 0
