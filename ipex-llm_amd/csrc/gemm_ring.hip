@@ -90,7 +90,7 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: LDS-DMA targets are scalars
     const int G = K / TILE_COLS;
     const int n_tiles = N / TILE_ROWS;
-    const int tiles_m = (M + 32 * MB - 1) / (32 * MB), tiles_n = (N + RN - 1) / RN;
+    const int tiles_m = (M + 32 * MB - 1) / (32 * MB);
     const int kg = lane >> 5, i32 = lane & 31, r16 = lane & 15;
     const int slot_lo = kg * 16 + r16, slot_hi = (kg + 2) * 16 + r16;
 
