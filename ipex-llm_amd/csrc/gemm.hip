@@ -83,18 +83,42 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
         // Grouped mode (mixture-of-experts): rows group_offsets[e] .. group_offsets[e+1]-1 of x use
         // weight group_weights[e].  The grid is sized on the host from an upper bound of row tiles;
         // every workgroup finds its group by walking the offsets (a handful of scalar loads).
-        const int mt = blockIdx.x % max_mtiles;
-        tile_n = blockIdx.x / max_mtiles;
-        int e = 0, base = 0, r0 = 0, r1 = 0;
+        // Whole row tiles first, then the groups' last, partly filled ones: the short tiles fill the
+        // gaps at the end of the launch instead of delaying whole tiles queued behind them.
+        int full = 0, part = 0;
+        for (int e = 0; e < n_groups; e++) {
+            const int rows = group_offsets[e + 1] - group_offsets[e];
+            full += rows / GM;
+            part += (rows % GM) != 0;
+        }
+        const int tiles_n = tn_cnt;
+        int idx;
+        bool want_full = true;
+        if ((int)blockIdx.x < full * tiles_n) {
+            idx = blockIdx.x % full;
+            tile_n = blockIdx.x / full;
+        } else {
+            const int b = blockIdx.x - full * tiles_n;
+            if (b >= part * tiles_n) return;                                        // whole workgroup leaves
+            want_full = false;
+            idx = b % part;
+            tile_n = b / part;
+        }
+        int e = 0, r0 = 0, r1 = 0;
         for (; e < n_groups; e++) {
             r0 = group_offsets[e];
             r1 = group_offsets[e + 1];
-            const int t = (r1 - r0 + GM - 1) / GM;
-            if (mt < base + t) break;
-            base += t;
+            const int f = (r1 - r0) / GM;
+            if (want_full) {
+                if (idx < f) break;
+                idx -= f;
+            } else if ((r1 - r0) % GM) {
+                if (idx == 0) { idx = f; break; }
+                idx--;
+            }
         }
-        if (e == n_groups) return;                                                  // whole workgroup leaves
-        m0 = r0 + (mt - base) * GM;
+        if (e == n_groups) return;
+        m0 = r0 + idx * GM;
         M = r1;                                     // rows past the group's end are clamped / not stored
         w = group_weights[e];
     }
