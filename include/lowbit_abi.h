@@ -271,6 +271,23 @@ int lowbit_gemm_ring(const void *x, const void *w, void *y, int qtype, int layou
 int lowbit_grouped_forward(const void *x, const void *const *w, void *y, const int32_t *group_offsets,
                            int n_groups, int64_t total_rows, int qtype, int act_dtype, int64_t N, int64_t K,
                            void *stream);
+/* The same with a workspace (caller-owned device memory, 16-byte aligned, lowbit_grouped_workspace_bytes(...)
+ * bytes; null / 0 is valid): when the output alone has too few tiles for the machine - few columns, long K, the
+ * down projection of an expert - K is split over a second grid dimension and the fp32 partial tiles are summed
+ * from the workspace by a second kernel.  lowbit_grouped_workspace_bytes returns 0 for shapes that do not split. */
+size_t lowbit_grouped_workspace_bytes(int n_groups, int64_t total_rows, int64_t N, int64_t K);
+int lowbit_grouped_forward_ws(const void *x, const void *const *w, void *y, const int32_t *group_offsets,
+                              int n_groups, int64_t total_rows, int qtype, int act_dtype, int64_t N, int64_t K,
+                              void *workspace, size_t workspace_bytes, void *stream);
+/* The gated MLP's first half for all experts in one launch: rows of group e of y [total_rows, N] =
+ * act(x w_gate[e]^T) .* (x w_up[e]^T), act as in lowbit_mlp_forward.  It is what the per-expert loop computes
+ * with two LowBitLinear calls and an activation per expert
+ * (python/llm/src/ipex_llm/transformers/models/qwen2_moe.py:375-430 calling the expert MLP of
+ * models/common.py:145-158), without the gate and up products ever leaving the registers.  w_gate / w_up /
+ * group_offsets as in lowbit_grouped_forward. */
+int lowbit_grouped_mlp_forward(const void *x, const void *const *w_gate, const void *const *w_up, void *y,
+                               const int32_t *group_offsets, int n_groups, int64_t total_rows, int qtype,
+                               int act_dtype, int64_t N, int64_t K, int act, void *stream);
 
 #ifdef __cplusplus
 }

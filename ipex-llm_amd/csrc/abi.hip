@@ -32,8 +32,10 @@ int gemm_splits(int M, int N, int K, size_t ws_bytes);
 double gemm_time_us(int M, int N, int K, int splits);
 int launch_gemv_bf16_f32out(const void *x, const void *w, void *y, int qtype, int layout, int M, int N, int K,
                             hipStream_t st);
-int launch_grouped_gemm(const void *x, const void *const *w, void *y, const int32_t *offsets, int n_groups,
-                        int total_rows, int qtype, int act_dtype, int N, int K, hipStream_t st);
+int launch_grouped_gemm(const void *x, const void *const *w, const void *const *w_up, void *y, const int32_t *offsets,
+                        int n_groups, int total_rows, int qtype, int act_dtype, int N, int K, int act, void *workspace,
+                        size_t workspace_bytes, hipStream_t st);
+size_t grouped_workspace_bytes(int total_rows, int n_groups, int N, int K);
 }  // namespace lowbit
 
 using namespace lowbit;
@@ -443,18 +445,48 @@ int lowbit_moe_forward(const void *x, const int32_t *topk_ids, const float *topk
                         "lowbit_moe_forward");
 }
 
+static int grouped_any(const char *who, const void *x, const void *const *w, const void *const *w_up, void *y,
+                       const int32_t *group_offsets, int n_groups, int64_t total_rows, int qtype, int act_dtype, int64_t N,
+                       int64_t K, int act, void *workspace, size_t workspace_bytes, void *stream) {
+    if (int rc = check_weight_shape(who, qtype, N, K, LOWBIT_LAYOUT_TILED)) return rc;
+    if (n_groups < 0 || total_rows < 0 || total_rows > 0x7fffffff)
+        return fail(LOWBIT_EARG, "%s: bad group count or row count", who);
+    if (act_dtype != LOWBIT_DT_F16 && act_dtype != LOWBIT_DT_BF16)
+        return fail(LOWBIT_EDTYPE, "%s: activations must be f16 or bf16", who);
+    if (act != LOWBIT_ACT_SILU && act != LOWBIT_ACT_GELU)
+        return fail(LOWBIT_EARG, "%s: activation must be LOWBIT_ACT_SILU or LOWBIT_ACT_GELU", who);
+    if (total_rows == 0 || n_groups == 0 || N == 0) return 0;
+    if (!x || !w || !y || !group_offsets || !aligned16(x) || (((uintptr_t)y) & 7) || (workspace && !aligned16(workspace)))
+        return fail(LOWBIT_EARG, "%s: null or misaligned pointer", who);
+    return check_launch(launch_grouped_gemm(x, w, w_up, y, group_offsets, n_groups, (int)total_rows, qtype, act_dtype, (int)N,
+                                            (int)K, act, workspace, workspace_bytes, (hipStream_t)stream), who);
+}
+
 int lowbit_grouped_forward(const void *x, const void *const *w, void *y, const int32_t *group_offsets, int n_groups,
                            int64_t total_rows, int qtype, int act_dtype, int64_t N, int64_t K, void *stream) {
-    if (int rc = check_weight_shape("lowbit_grouped_forward", qtype, N, K, LOWBIT_LAYOUT_TILED)) return rc;
-    if (n_groups < 0 || total_rows < 0 || total_rows > 0x7fffffff)
-        return fail(LOWBIT_EARG, "lowbit_grouped_forward: bad group count or row count");
-    if (act_dtype != LOWBIT_DT_F16 && act_dtype != LOWBIT_DT_BF16)
-        return fail(LOWBIT_EDTYPE, "lowbit_grouped_forward: activations must be f16 or bf16");
-    if (total_rows == 0 || n_groups == 0 || N == 0) return 0;
-    if (!x || !w || !y || !group_offsets || !aligned16(x) || (((uintptr_t)y) & 7))
-        return fail(LOWBIT_EARG, "lowbit_grouped_forward: null or misaligned pointer");
-    return check_launch(launch_grouped_gemm(x, w, y, group_offsets, n_groups, (int)total_rows, qtype, act_dtype, (int)N,
-                                            (int)K, (hipStream_t)stream), "lowbit_grouped_forward");
+    return grouped_any("lowbit_grouped_forward", x, w, nullptr, y, group_offsets, n_groups, total_rows, qtype, act_dtype, N, K,
+                       LOWBIT_ACT_SILU, nullptr, 0, stream);
+}
+
+size_t lowbit_grouped_workspace_bytes(int n_groups, int64_t total_rows, int64_t N, int64_t K) {
+    if (n_groups <= 0 || total_rows <= 0 || total_rows > 0x7fffffff || N <= 0 || K <= 0 || N > 0x7fffffff || K > 0x7fffffff)
+        return 0;
+    return grouped_workspace_bytes((int)total_rows, n_groups, (int)N, (int)K);
+}
+
+int lowbit_grouped_forward_ws(const void *x, const void *const *w, void *y, const int32_t *group_offsets, int n_groups,
+                              int64_t total_rows, int qtype, int act_dtype, int64_t N, int64_t K, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+    return grouped_any("lowbit_grouped_forward_ws", x, w, nullptr, y, group_offsets, n_groups, total_rows, qtype, act_dtype, N,
+                       K, LOWBIT_ACT_SILU, workspace, workspace_bytes, stream);
+}
+
+int lowbit_grouped_mlp_forward(const void *x, const void *const *w_gate, const void *const *w_up, void *y,
+                               const int32_t *group_offsets, int n_groups, int64_t total_rows, int qtype, int act_dtype,
+                               int64_t N, int64_t K, int act, void *stream) {
+    if (!w_up) return fail(LOWBIT_EARG, "lowbit_grouped_mlp_forward: null pointer");
+    return grouped_any("lowbit_grouped_mlp_forward", x, w_gate, w_up, y, group_offsets, n_groups, total_rows, qtype, act_dtype,
+                       N, K, act, nullptr, 0, stream);
 }
 
 }  // extern "C"

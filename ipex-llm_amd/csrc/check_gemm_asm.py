@@ -1,0 +1,154 @@
+#!/usr/bin/env python3
+"""Checks the generated assembly of the MFMA GEMM kernels for what the compiler cannot know.
+
+The v_mfma_f32_32x32x16 instructions of lowbit_gemm.h sit in inline assembly, so the compiler neither knows
+that their results arrive late (18 wait states for a 16-pass MFMA) nor that they are MFMAs at all.  The source
+keeps every accumulator block in one place from the first MFMA to the epilogue; this script verifies that the
+compiler went along with it, per kernel of an assembly listing (hipcc -S --cuda-device-only):
+
+  1. every read of an accumulation register that an MFMA writes (v_accvgpr_read, the source of a v_accvgpr_mov,
+     a store straight from accumulation registers) comes at least MIN_WAIT wait states after the nearest MFMA
+     ahead of it in program order that writes that register - the compiler does move accumulator blocks between
+     registers where variants of the main loop meet, which is harmless for a block whose MFMA is long done and
+     loses a K step for the block written last;
+  2. no such register is overwritten (v_accvgpr_mov, v_accvgpr_write) that soon after its MFMA either;
+  3. the kernel uses no scratch memory and calls no function (a variant of the main loop that is not inlined
+     keeps its closure in scratch and reads the weights with flat loads);
+  4. no LDS-DMA takes its scalar base address from a v_readfirstlane less than 5 wait states earlier (VALU
+     write of an SGPR followed by a VMEM read of it).
+
+usage: check_gemm_asm.py listing.s [--allow-scratch SUBSTRING ...]
+Exit status 0 when every kernel passes, 1 otherwise.
+"""
+import re
+import sys
+
+MIN_WAIT = 18
+
+
+def instructions(lines):
+    for no, line in enumerate(lines):
+        t = line.strip()
+        if not t or t.startswith((";", ".", "//")) or t.endswith(":"):
+            continue
+        yield no, t
+
+
+def wait_states(t):
+    """Cycles an instruction keeps the wave busy at the least.  Another MFMA cannot issue before the one ahead of
+    it has gone through its 8 passes of 4 cycles: whatever comes after a later MFMA is safe."""
+    m = re.match(r"s_nop (\d+)", t)
+    if m:
+        return int(m.group(1)) + 1
+    return 32 if t.startswith("v_mfma_f32_32x32x16") else 1
+
+
+def regs(spec):
+    """'a[4:7]' or 'a5' -> set of register numbers."""
+    m = re.match(r"a\[(\d+):(\d+)\]", spec)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"a(\d+)$", spec)
+    return {int(m.group(1))} if m else set()
+
+
+def check_kernel(name, lines, allow_scratch, first_line=0):
+    errors = []
+    ins = [(no + first_line, t) for no, t in instructions(lines)]
+    mfma_dst = set()
+    mfma_at = []
+    for k, (no, t) in enumerate(ins):
+        m = re.match(r"v_mfma_\S+ (a\[\d+:\d+\])", t)
+        if m:
+            mfma_dst |= regs(m.group(1))
+            mfma_at.append(k)
+    if not mfma_at:
+        return errors
+    mfma_writes = {}
+    for k in mfma_at:
+        mfma_writes[k] = regs(re.match(r"v_mfma_\S+ (a\[\d+:\d+\])", ins[k][1]).group(1))
+
+    def since_write(k, wanted):
+        """Wait states between the nearest MFMA ahead of instruction k (in program order, up to an unconditional
+        branch) that writes one of `wanted` and instruction k; MIN_WAIT if there is none that close."""
+        w = 0
+        for j in range(k - 1, -1, -1):
+            t = ins[j][1]
+            if j in mfma_writes and (mfma_writes[j] & wanted):
+                return w
+            if re.match(r"s_branch|s_endpgm|s_setpc_b64", t):
+                break
+            w += wait_states(t)
+            if w >= MIN_WAIT:
+                break
+        return MIN_WAIT
+
+    for k, (no, t) in enumerate(ins):
+        read = set()
+        m = re.match(r"v_accvgpr_mov_b32 a\d+, (a\d+)", t)
+        if m:
+            read = regs(m.group(1))
+        m = re.match(r"v_accvgpr_read_b32 v\d+, (a\d+)", t)
+        if m:
+            read = regs(m.group(1))
+        m = re.match(r"(?:global|flat|scratch|buffer)_store\S* .*?(a\[\d+:\d+\]|a\d+)", t)
+        if m:
+            read = regs(m.group(1))
+        if read & mfma_dst:
+            w = since_write(k, read)
+            if w < MIN_WAIT:
+                errors.append(f"line {no + 1}: accumulator read {w} wait states after the MFMA that writes it: {t}")
+        # overwriting a block while its MFMA is still in flight loses the result just the same
+        m = re.match(r"v_accvgpr_(?:mov|write)_b32 (a\d+),", t)
+        if m and (regs(m.group(1)) & mfma_dst):
+            w = since_write(k, regs(m.group(1)))
+            if w < MIN_WAIT:
+                errors.append(f"line {no + 1}: accumulator overwritten {w} wait states after the MFMA that writes it: {t}")
+        if re.match(r"s_swappc_b64|s_call_b64", t):
+            errors.append(f"line {no + 1}: function call: {t}")
+        if t.startswith("scratch_") and not any(a in name for a in allow_scratch):
+            errors.append(f"line {no + 1}: scratch access: {t}")
+            break
+        m = re.match(r"global_load_lds_dwordx4 v\d+, s\[(\d+):(\d+)\]", t)
+        if m:
+            base = {int(m.group(1)), int(m.group(2))}
+            w = 0
+            for j in range(k - 1, -1, -1):
+                mm = re.match(r"v_readfirstlane_b32 s(\d+),", ins[j][1])
+                if mm and int(mm.group(1)) in base:
+                    errors.append(f"line {no + 1}: LDS-DMA base written by VALU {w} wait states earlier")
+                    break
+                w += wait_states(ins[j][1])
+                if w >= 5:
+                    break
+    return errors
+
+
+def main(argv):
+    if len(argv) < 2:
+        print(__doc__)
+        return 2
+    allow = []
+    if "--allow-scratch" in argv:
+        i = argv.index("--allow-scratch")
+        allow = argv[i + 1:]
+        argv = argv[:i]
+    text = open(argv[1]).read().split("\n")
+    starts = [i for i, l in enumerate(text) if re.match(r"_Z\w+:\s", l + " ")]
+    bad = 0
+    for n, s in enumerate(starts):
+        name = text[s].split(":")[0]
+        if "gemm_mfma_kernel" not in name:
+            continue
+        e = starts[n + 1] if n + 1 < len(starts) else len(text)
+        errors = check_kernel(name, text[s:e], allow, s)
+        label = "ok" if not errors else f"{len(errors)} problem(s)"
+        print(f"{name}: {label}")
+        for msg in errors[:10]:
+            print("   ", msg)
+        bad += bool(errors)
+    return 1 if bad else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv))

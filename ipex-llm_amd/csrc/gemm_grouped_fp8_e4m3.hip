@@ -1,0 +1,9 @@
+// The grouped GEMM kernels (lowbit_gemm_grouped.h) for fp8_e4m3 weights.
+#include "lowbit_gemm_grouped.h"
+
+namespace lowbit {
+
+template int launch_grouped_q<QT_FP8_E4M3>(const void *, const void *const *, const void *const *, void *, const int32_t *, int, int,
+                                    int, int, int, int, const GroupedPlan &, float *, hipStream_t);
+
+}  // namespace lowbit

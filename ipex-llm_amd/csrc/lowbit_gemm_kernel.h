@@ -1,0 +1,588 @@
+// The tiled MFMA GEMM kernel, shared by the dense launchers (gemm.hip) and the grouped ones for
+// mixture-of-experts layers (gemm_grouped.hip).
+//
+// Workgroup tile: 128 rows of x (M) by 256 weight rows (N), 4 waves side by side along N,
+// so that every weight is dequantized by exactly one wave.  Per 128-column step of K:
+//   weights: each lane loads its 16/32 bytes of four tiles straight from HBM into registers -
+//            the tiled layout already is the MFMA operand layout - and turns them into scaled
+//            fp16 / bf16 values in registers (no LDS for weights);
+//   x:       the workgroup copies the 128 x 128 block of x into LDS in operand order
+//            (double buffered), and every wave reads it from there;
+//   8 v_mfma_f32_32x32x16 per 16 columns and wave, weights as the A operand (rows = n) and x
+//   as the B operand (columns = m), so a lane ends up with groups of 4 consecutive n for one m
+//   and stores 8 contiguous bytes of y at a time.
+#pragma once
+#include "lowbit_gemm.h"
+
+namespace lowbit {
+
+constexpr int GM = 128;          // rows of x per workgroup (the tall form below takes 256)
+constexpr int GN_WAVE = 64;      // weight rows per wave
+constexpr int GN = 256;          // weight rows per workgroup (4 waves)
+
+constexpr int MB32 = GM / 32;        // 32-row blocks of x per workgroup
+constexpr int NB32 = GN_WAVE / 32;   // 32-row blocks of W per wave (two tiles each)
+constexpr int GM_TALL = 256, MB32_TALL = GM_TALL / 32;
+
+// Operand layout of v_mfma_f32_32x32x16: lane l = 32*kg + i holds 8 consecutive k (8*kg .. +7 of
+// the 16-column step) of row/column i.  A 32-row weight block is two tiles (rows 0-15, 16-31);
+// in a tile, lane slot 16*c + r holds columns 8*c .. +7 of each 32-column sub-block, so lane
+// (kg, i) takes slot 16*kg + i%16 of tile i/16 for the first 16 columns of every sub-block
+// ("lo" registers) and slot 16*(kg+2) + i%16 for the second 16 columns ("hi" registers).
+//
+// MB = 32-row blocks of x per workgroup: 4 (128 rows) or, for the tall form, 8 (256 rows, DMA form only).  The
+// tall form dequantizes every weight once per 256 rows of x: half the VALU work, half the weight loads and
+// half the barriers per MFMA; its 16 accumulator blocks take all 256 accumulation registers, so a CU holds
+// one workgroup.  tn0 / tn_cnt: the launch covers the column tiles tn0 .. tn0 + tn_cnt - 1 of y.
+// Grouped mode (mixture-of-experts): rows offsets[e] .. offsets[e+1]-1 of x use the weight w[e]
+// (and w_up[e] in the fused gate/up form); all pointers are device memory.
+struct GroupArgs {
+    const int32_t *offsets;
+    const uint8_t *const *w;
+    const uint8_t *const *w_up;
+    int n_groups;
+    int act;                      // activation of the gate branch in the fused form: 0 = SiLU, 1 = tanh-GELU
+};
+
+// Which row tile of which group workgroup `b` of a grouped launch works on.  Whole row tiles come first, then
+// the groups' last, partly filled ones: the short tiles fill the gaps at the end of the launch instead of
+// delaying whole tiles queued behind them, and no idle workgroup sits between working ones (workgroups go to
+// the compute units of an XCD in turn: with every other workgroup leaving at once, half of the units idled).
+// The partly filled tiles of a column go to the XCDs (workgroup id % 8) in an order that rotates from column
+// to column: with eight groups each XCD would otherwise work on one group only and the XCD of the group with
+// the most rows would finish last (measured with 10 to 300 rows per group: 9-12 % of the launch).
+struct GroupTile {
+    int group, m0, m_end, tile_n;
+};
+template <int ROWS>
+__device__ inline bool grouped_tile(const int32_t *__restrict__ offsets, int n_groups, int tiles_n, int b, GroupTile &t) {
+    int full = 0, part = 0;
+    for (int e = 0; e < n_groups; e++) {
+        const int rows = offsets[e + 1] - offsets[e];
+        full += rows / ROWS;
+        part += (rows % ROWS) != 0;
+    }
+    int idx;
+    bool want_full = true;
+    if (b < full * tiles_n) {
+        idx = b % full;
+        t.tile_n = b / full;
+    } else {
+        b -= full * tiles_n;
+        if (b >= part * tiles_n) return false;
+        want_full = false;
+        t.tile_n = b / part;
+        idx = (b + t.tile_n) % part;
+    }
+    for (int e = 0; e < n_groups; e++) {
+        const int r0 = offsets[e], r1 = offsets[e + 1];
+        const int f = (r1 - r0) / ROWS;
+        if (want_full) {
+            if (idx < f) { t.group = e; t.m0 = r0 + idx * ROWS; t.m_end = r1; return true; }
+            idx -= f;
+        } else if ((r1 - r0) % ROWS) {
+            if (idx == 0) { t.group = e; t.m0 = r0 + f * ROWS; t.m_end = r1; return true; }
+            idx--;
+        }
+    }
+    return false;
+}
+
+// A 64-bit value that is the same in every lane, moved to scalar registers.  (The builtin returns a signed
+// int: each half goes through uint32_t on its way back, or the low half would sign-extend into the high one.)
+__device__ inline uint64_t uniform64(uint64_t v) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (uint64_t)lo | ((uint64_t)hi << 32);
+}
+
+// activation of the gate branch: 0 = SiLU, 1 = GELU in its tanh form
+__device__ inline float gemm_gate_act(float g, int act) {
+    if (act == 0) return g / (1.0f + __expf(-g));
+    const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
+    return 0.5f * g * (1.0f + t);
+}
+
+// GROUPED: the launch covers the row tiles of all groups (see GroupArgs); the tall form then takes one row
+// tile for up to 256 rows of a group and runs only the 32-row blocks that hold rows.
+// DUAL (grouped tall form only): the fused gate/up projection of a gated MLP.  The wave's two 32-row weight
+// blocks are the same 32 rows of the gate and of the up weight (a workgroup covers 128 columns of both), and
+// the epilogue stores act(gate) * up.
+template <int QT, typename AT, bool DMA, int MB, bool GROUPED = false, bool DUAL = false>
+__global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+                                                        AT *__restrict__ y, int M, int N, int K, int xcd_m,
+                                                        const GroupArgs ga, int k_steps,
+                                                        float *__restrict__ ws, int tn0, int tn_cnt) {
+    using F = Fmt<QT>;
+    using V8 = typename Vec8<AT>::type;
+    static_assert(MB == 4 || (MB == 8 && DMA), "row tiles of 128 rows, or 256 rows in the DMA form");
+    static_assert(!DUAL || (GROUPED && MB == 8), "the fused gate/up form exists for grouped launches of the tall form");
+    constexpr int MB32 = MB, GM = 32 * MB;            // shadow the 128-row constants of the file
+    // x block of a K step: 8 * MB32 pieces of 1 KiB (layout below), double buffered
+    __shared__ __attribute__((aligned(16))) uint8_t xs0[8 * MB32 * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t xs1[8 * MB32 * 1024];
+    __shared__ float lut[16];
+    if constexpr (QT == QT_NF4) {
+        if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODEBOOK[threadIdx.x];
+    }
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: scalar address arithmetic
+    const int G = K / TILE_COLS;
+    const int n_tiles = N / TILE_ROWS;
+
+    // Workgroups are handed to the 8 XCDs round-robin (id % 8) and each XCD has its own L2.  The
+    // output tiles are therefore dealt out so that one XCD owns a block of band_m row-tiles by
+    // band_n column-tiles: its L2 then only has to hold that band of x (re-read by every
+    // column-tile) and sees each weight tile from all its row-tiles at about the same time.
+    int m0, tile_n;
+    const uint8_t *w_up = nullptr;
+    if constexpr (!GROUPED) {
+        const int tiles_m = (M + GM - 1) / GM, tiles_n = tn_cnt;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        const int band_m = (tiles_m + xcd_m - 1) / xcd_m;
+        const int xcd_n = 8 / xcd_m;
+        const int band_n = (tiles_n + xcd_n - 1) / xcd_n;
+        const int tile_m = (xcd % xcd_m) * band_m + slot % band_m;
+        tile_n = (xcd / xcd_m) * band_n + slot / band_m;
+        if (slot >= band_m * band_n || tile_m >= tiles_m || tile_n >= tiles_n) return;   // whole workgroup leaves
+        tile_n += tn0;
+        m0 = tile_m * GM;
+    } else {
+        // every workgroup finds its group by walking the offsets (a handful of scalar loads)
+        GroupTile gt;
+        if (!grouped_tile<GM>(ga.offsets, ga.n_groups, tn_cnt, blockIdx.x, gt)) return;    // whole workgroup leaves
+        // (the compiler does not see that what comes out of the walk is the same in every lane)
+        tile_n = __builtin_amdgcn_readfirstlane(gt.tile_n);
+        m0 = __builtin_amdgcn_readfirstlane(gt.m0);
+        M = __builtin_amdgcn_readfirstlane(gt.m_end);   // rows past the group's end are clamped / not stored
+        const int group = __builtin_amdgcn_readfirstlane(gt.group);
+        w = ga.w[group];
+        if constexpr (DUAL) w_up = ga.w_up[group];
+    }
+    constexpr int GN_WG = DUAL ? GN / 2 : GN, GN_W = DUAL ? GN_WAVE / 2 : GN_WAVE;   // columns of y per workgroup, per wave
+    const int n0 = tile_n * GN_WG + wave * GN_W;
+
+    // weight tiles of this lane: block nb covers rows n0 + 32*nb .. +31 (clamped: a tile row past N
+    // is computed and never stored)
+    const int kg = lane >> 5, i32 = lane & 31, r16 = lane & 15;
+    const int slot_lo = kg * 16 + r16, slot_hi = (kg + 2) * 16 + r16;
+    gbytes wt[NB32];
+#pragma unroll
+    for (int nb = 0; nb < NB32; nb++) {
+        int trow = n0 / TILE_ROWS + (DUAL ? 0 : nb * 2) + (i32 >> 4);
+        trow = trow < n_tiles ? trow : n_tiles - 1;
+        wt[nb] = (gbytes)((DUAL && nb == 1) ? w_up : w) + (int64_t)trow * G * F::TILE_BYTES;
+    }
+
+    // The x block of a K step (128 rows x 256 bytes) sits in LDS as 32 pieces of 1 KiB: piece h * 16 + t
+    // holds rows 8t .. 8t+7 of the half row h (64 columns = 128 bytes), the 16 bytes of (row r, 16-byte
+    // chunk c) at (c * 8 + r % 8) * 16.  Lane (kg, i) of the MFMA reads, for 16-column step ks and row
+    // block mb, piece (ks/4) * 16 + 4*mb + i/8 at ((ks%4 * 2 + kg) * 8 + i%8) * 16: eight consecutive
+    // lanes read 128 contiguous bytes.  The layout is chosen for the DMA form below.
+    //
+    // Register-staged form: x goes global -> registers -> LDS; a wave-wide load covers 16 rows x 64
+    // bytes: chunk = 4*wave + lane/16 (16 bytes each), row = 16*i + lane%16 for i = 0..7.
+    const int chunk = wave * 4 + (lane >> 4);
+    uint32_t xoff[DMA ? 1 : 8];
+    int xl[DMA ? 1 : 8];
+    // DMA form: x goes global -> LDS without passing through registers.  One wave-wide instruction
+    // fills one piece: lane 8*c + i fetches the 16 bytes at row 8t + i, byte 16c of the half row - whole
+    // 128-byte lines, 8 per instruction - and the hardware writes the lanes to LDS in lane order.  Wave
+    // w fills pieces 8w .. 8w+7: half row w/2, rows 64*(w%2) + 8j + i.  Rows past M are clamped (the
+    // offsets are formed with 24-bit multiplies: the launcher keeps M and 2K below 2^24).
+    uint32_t xrow0 = 0, xcol = 0;
+    if constexpr (!DMA) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int row_in = i * 16 + r16;
+            int row = m0 + row_in;
+            row = row < M ? row : M - 1;
+            xoff[i] = (uint32_t)(((int64_t)row * K + chunk * 8) * (int64_t)sizeof(AT));
+            xl[i] = (((chunk >> 3) * (4 * MB32) + (row_in >> 3)) * 64 + (chunk & 7) * 8 + (row_in & 7)) * 16;
+        }
+    } else {
+        xrow0 = m0 + (GM / 2) * (wave & 1) + (lane & 7);
+        xcol = (wave >> 1) * 128 + (lane >> 3) * 16;
+    }
+    constexpr int PW = 2 * MB32;                     // pieces of 1 KiB (8 rows of a half row) a wave fetches per K step
+    // Split-K: with a workspace the grid has a second dimension, workgroup (t, s) walks the K steps
+    // s * k_steps .. and leaves its fp32 partial tile in ws[s]; a second kernel sums the splits.  It
+    // fills the machine when the output alone has too few tiles (small M, narrow N).
+    const int kt0 = ws ? blockIdx.y * k_steps : 0;
+    const int Gs = ws ? (k_steps < G - kt0 ? k_steps : G - kt0) : G;
+    const int last = Gs - 1;
+    // the same loads one at a time, for spreading them over a step: a burst of 8 + 6 loads per wave,
+    // from eight waves at once, queues up at the CU's address unit and the waves stand still meanwhile
+    // (measured with cycle counters: 41 % of a K step at M = 2048)
+    auto dma_x_one = [&](int kt, uint8_t *buf, int j) __attribute__((always_inline)) {
+        kt = kt0 + (kt < last ? kt : last);
+        // Issued from inline assembly: the compiler's wait-count pass treats an LDS-DMA as aliasing
+        // every later LDS access and would wait for it immediately.  Completion is awaited by the
+        // explicit vmcnt(0) ahead of the workgroup barrier that publishes the buffer.
+        const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
+        const uint32_t lbase = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + wave * PW * 1024);
+        uint32_t row = xrow0 + 8 * j;
+        row = row < (uint32_t)M ? row : (uint32_t)M - 1;
+        const uint8_t *src = xk + (__umul24(row, (uint32_t)K * (uint32_t)sizeof(AT)) + xcol);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :: "v"(src), "s"(lbase + j * 1024) : "memory", "m0");
+    };
+    // Tall form: the per-lane part of the address is a constant 32-bit offset and everything that changes from
+    // load to load is scalar arithmetic.  Dense launches hand it whole 256-row tiles only, so no row is clamped.
+    const uint32_t xlane_off = (uint32_t)(lane & 7) * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)(lane >> 3) * 16u;
+    const uint64_t xwave_base = (uint64_t)(uintptr_t)x +
+        ((uint64_t)(m0 + (GM / 2) * (wave & 1)) * (uint64_t)K + (uint64_t)(wave >> 1) * 64u) * sizeof(AT);
+    auto dma_x_scalar = [&](int kt, uint8_t *buf, int j) __attribute__((always_inline)) {
+        kt = kt0 + (kt < last ? kt : last);
+        const uint64_t src = xwave_base + (uint64_t)kt * (TILE_COLS * sizeof(AT)) + (uint64_t)j * 8u * (uint64_t)K * sizeof(AT);
+        const uint32_t lbase = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + (wave * PW + j) * 1024);
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(xlane_off), "s"(src), "s"(lbase) : "memory", "m0");
+    };
+    // Grouped tall form: a tile holds rows_here <= 256 rows of its group and only the first MBC 32-row blocks are
+    // computed.  Wave w fills the pieces 2j + w % 2 (rows 8 * (2j + w % 2) ..) of half row w / 2 for j < 2 * MBC:
+    // the same count for every wave and a bound known at compile time, so that the main loop stays free of
+    // branches.  The two pieces of the last block may reach past the group's rows: they take their rows from a
+    // per-lane offset relative to the tile's first row, with the row clamped to the group's last one (rows past
+    // it are computed from a copy of that row and never stored).
+    const int rows_here = __builtin_amdgcn_readfirstlane(M - m0 < GM ? M - m0 : GM);
+    uint64_t xtile_base = (uint64_t)(uintptr_t)x + ((uint64_t)m0 * (uint64_t)K + (uint64_t)(wave >> 1) * 64u) * sizeof(AT);
+    auto tail_offset = [&](int j) __attribute__((always_inline)) {            // piece j of this wave, rows clamped
+        int row = 8 * (2 * j + (wave & 1)) + (lane & 7);
+        row = row < rows_here ? row : rows_here - 1;
+        return (uint32_t)row * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)(lane >> 3) * 16u;
+    };
+    auto dma_x_grouped = [&](int kt, uint8_t *buf, int j, auto mbc_, const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
+        constexpr int MBC = decltype(mbc_)::value;
+        kt = kt0 + (kt < last ? kt : last);
+        const bool tail = j >= 2 * (MBC - 1);
+        uint64_t src = xtile_base + (uint64_t)kt * (TILE_COLS * sizeof(AT));
+        if (!tail) src += (uint64_t)(8 * (2 * j + (wave & 1))) * (uint64_t)K * sizeof(AT);
+        // the same in every lane, which the compiler does not always see after the walk over the groups
+        src = uniform64(src);
+        const uint32_t lbase = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + ((wave >> 1) * (4 * MB32) + 2 * j + (wave & 1)) * 1024);
+        const uint32_t voff = tail ? voff_tail[j - 2 * (MBC - 1) < 0 ? 0 : j - 2 * (MBC - 1)] : xlane_off;
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(voff), "s"(src), "s"(lbase) : "memory", "m0");
+    };
+    constexpr bool GTALL = GROUPED && MB32 == 8;
+    auto dma_x = [&](int kt, uint8_t *buf, auto mbc_, const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < (GTALL ? 2 * decltype(mbc_)::value : PW); j++) {
+            if constexpr (GTALL) dma_x_grouped(kt, buf, j, mbc_, voff_tail);
+            else if constexpr (MB32 == 8) dma_x_scalar(kt, buf, j);
+            else dma_x_one(kt, buf, j);
+        }
+    };
+    auto load_x = [&](int kt, u32x4 (&xr)[8]) __attribute__((always_inline)) {
+        kt = kt0 + (kt < last ? kt : last);              // past the end: a harmless re-read, never used
+        const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
+#pragma unroll
+        for (int i = 0; i < 8; i++) xr[i] = *(const u32x4 *)(xk + xoff[i]);
+    };
+    auto load_x_one = [&](int kt, u32x4 (&xr)[8], int i) __attribute__((always_inline)) {
+        kt = kt0 + (kt < last ? kt : last);
+        xr[i] = *(const u32x4 *)((const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT) + xoff[DMA ? 0 : i]);
+    };
+    auto store_x = [&](uint8_t *buf, const u32x4 (&xr)[8]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) *(u32x4 *)(buf + xl[i]) = xr[i];
+    };
+    struct WRegs {
+        TileRegs<QT> lo[NB32], hi[NB32];
+    };
+    auto load_w = [&](int kt, WRegs &t) __attribute__((always_inline)) {
+        kt = kt0 + (kt < last ? kt : last);
+#pragma unroll
+        for (int nb = 0; nb < NB32; nb++) {
+            const gbytes tile = wt[nb] + (int64_t)kt * F::TILE_BYTES;
+            load_tile<QT>(tile, slot_lo, r16, t.lo[nb]);
+            t.hi[nb].q0 = ld<u32x4>(tile + slot_hi * 16);
+            if constexpr (F::BITS == 8) t.hi[nb].q1 = ld<u32x4>(tile + 1024 + slot_hi * 16);
+        }
+    };
+
+    auto load_w_nb = [&](int kt, WRegs &t, int nb) __attribute__((always_inline)) {
+        kt = kt0 + (kt < last ? kt : last);
+        const gbytes tile = wt[nb] + (int64_t)kt * F::TILE_BYTES;
+        load_tile<QT>(tile, slot_lo, r16, t.lo[nb]);
+        t.hi[nb].q0 = ld<u32x4>(tile + slot_hi * 16);
+        if constexpr (F::BITS == 8) t.hi[nb].q1 = ld<u32x4>(tile + 1024 + slot_hi * 16);
+    };
+
+    // The loads of the next K step, as NB32 + PW units (the weight registers of a 32-row block; one piece of x),
+    // dealt out over the first five eighths of the step's MFMA groups, so that the data has the rest of the
+    // step to arrive and no group carries more than a load or two: a burst stalls the waves at the CU's
+    // address unit (41 % of a K step at M = 2048 when all loads of a step went out together), and with one or
+    // two waves per SIMD every cycle a wave stands at a memory instruction is a cycle its MFMA pipe idles.
+    // `point` = index of the MFMA group (16-column step * row blocks + row block) the call follows.
+    auto fetch_units = [&](int kt, uint8_t *buf, WRegs &t, const int point, const int points, auto mbc_,
+                           const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
+        constexpr int UNITS = NB32 + (GTALL ? 2 * decltype(mbc_)::value : PW);
+        const int spread = points * 5 / 8 > 0 ? points * 5 / 8 : 1;
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            if (u < point * UNITS / spread || u >= (point + 1) * UNITS / spread || point >= spread) continue;
+            if (u < NB32) load_w_nb(kt, t, u);
+            else if constexpr (GTALL) dma_x_grouped(kt, buf, u - NB32, mbc_, voff_tail);
+            else if constexpr (MB32 == 8) dma_x_scalar(kt, buf, u - NB32);
+            else dma_x_one(kt, buf, u - NB32);
+        }
+    };
+
+    // One set of accumulators for all variants of the main loop, cleared here.  Every MFMA names its
+    // accumulator as an in-out operand of its assembly statement, which keeps each block in the same accumulation
+    // registers from here to the epilogue.  It has to: the compiler does not know that the statements are MFMAs
+    // and would copy a block to other registers without the wait states a fresh MFMA result needs.  (With the
+    // accumulators declared per variant it did: the last K step was lost.  check_gemm_asm.py looks for such
+    // copies in the generated assembly.)
+    f32x16 acc[MB32][NB32];
+#pragma unroll
+    for (int mb = 0; mb < MB32; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB32; nb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[mb][nb][i] = 0.0f;
+
+    const DqCtx ctx = {lut, dq_magic<QT, AT>()};
+    // weights of 16-column step ks for block nb: sub-block ks/2, lo or hi registers
+    auto dequant_pair = [&](const WRegs &t, int ks, int nb, int p) __attribute__((always_inline)) -> uint32_t {
+        if (ks & 1) {
+            TileRegs<QT> h = t.hi[nb];
+            h.h = t.lo[nb].h;
+            return Dequant<QT, AT>::pair(h, ks >> 1, p, ctx);
+        }
+        return Dequant<QT, AT>::pair(t.lo[nb], ks >> 1, p, ctx);
+    };
+
+    // 8 steps of 16 columns, written in the order the hardware should issue them: after the MFMAs
+    // of an m-block its x operand for the NEXT step is requested from LDS, and register pairs of
+    // the next step's weights are dequantized after every MFMA, so that LDS latency and the VALU
+    // work run in the shadow of the MFMA pipe.  MBC = number of 32-row blocks of x that take part
+    // (a compile-time constant: a branch around each MFMA would cut the schedule into pieces).
+    auto x_piece = [](int ks, int mb) __attribute__((always_inline)) { return ((ks / 4) * 4 * MB32 + 4 * mb) * 1024 + (ks % 4) * 256; };
+    const int xlane = (i32 >> 3) * 1024 + kg * 128 + (i32 & 7) * 16;
+    auto compute = [&](auto &acc, const uint8_t *cur, const WRegs &t, auto mbc_, auto &&between) __attribute__((always_inline)) {
+        constexpr int MBC = decltype(mbc_)::value;
+        constexpr int SLOTS = MBC * NB32, PAIRS = 4 * NB32;   // MFMAs per 16-column step; register pairs to dequantize meanwhile
+        V8 xv[MBC];
+        u32x4 wv[NB32];
+#pragma unroll
+        for (int mb = 0; mb < MBC; mb++) xv[mb] = *(const V8 *)(cur + xlane + x_piece(0, mb));
+#pragma unroll
+        for (int nb = 0; nb < NB32; nb++)
+#pragma unroll
+            for (int p = 0; p < 4; p++) wv[nb][p] = dequant_pair(t, 0, nb, p);
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            u32x4 wn[NB32];
+#pragma unroll
+            for (int mb = 0; mb < MBC; mb++) {
+#pragma unroll
+                for (int nb = 0; nb < NB32; nb++) {
+                    mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    if (ks < 7) {
+                        // pairs [slot * PAIRS / SLOTS, (slot + 1) * PAIRS / SLOTS): spread evenly over the MFMA slots
+                        const int slot_i = mb * NB32 + nb;
+#pragma unroll
+                        for (int idx = 0; idx < PAIRS; idx++) {
+                            if (idx < slot_i * PAIRS / SLOTS || idx >= (slot_i + 1) * PAIRS / SLOTS) continue;
+                            wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);   // (weight block, pair)
+                        }
+                    }
+                }
+                if (ks < 7) xv[mb] = *(const V8 *)(cur + xlane + x_piece(ks + 1, mb));
+                // keep this order: the scheduler does not know how long an MFMA takes and would
+                // sink the LDS read down to its first use, exposing the LDS latency every time
+                __builtin_amdgcn_sched_barrier(0);
+                between(ks * MBC + mb, 8 * MBC);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (ks < 7) {
+#pragma unroll
+                for (int nb = 0; nb < NB32; nb++) wv[nb] = wn[nb];
+            }
+        }
+        // Where variants of the main loop meet, the compiler may move an accumulator block to other registers, and
+        // it does not know that the block written last is still in the MFMA pipe: leave it the time to land (the
+        // wave is on its way to a barrier here, the wait is hidden behind it).
+        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 1" : "+a"(acc[MBC - 1][NB32 - 1]));
+    };
+    typedef std::integral_constant<int, MB32> full_t;
+    auto nothing = [](int, int) __attribute__((always_inline)) {};
+
+    auto epilogue = [&](auto &acc, auto mbc_) __attribute__((always_inline)) {
+        constexpr int MBC = decltype(mbc_)::value;
+    // The MFMAs above are opaque to the compiler's hazard tracking: give the last results time to
+    // land before the accumulation registers are read back (a 16-pass MFMA needs 18 wait states
+    // before its result may be read; 64 are spent).  The accumulators are operands of the statement,
+    // so that no read of them can be scheduled ahead of it.
+#pragma unroll
+    for (int mb = 0; mb < MBC; mb++)
+        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7"
+                     : "+a"(acc[mb][0]), "+a"(acc[mb][1]));
+    // C layout of the 32x32 block: lane = 32*g + col (col = x row within the block), register i =
+    // weight row 8*(i/4) + 4*g + i%4: four consecutive n per group of registers
+#pragma unroll
+    for (int mb = 0; mb < MBC; mb++) {
+        const int m = m0 + mb * 32 + i32;
+        if constexpr (DUAL) {
+            // both blocks hold the same 32 columns of y: the gate branch in block 0, the up branch in block 1
+            if (m < M) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int n = n0 + q * 8 + kg * 4;
+                    if (n < N) {
+                        typedef AT at4 __attribute__((ext_vector_type(4)));
+                        at4 o;
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            o[i] = to_at<AT>(gemm_gate_act(acc[mb][0][q * 4 + i], ga.act) * acc[mb][1][q * 4 + i]);
+                        *(at4 *)(y + (int64_t)m * N + n) = o;
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        } else if (m < M) {
+#pragma unroll
+            for (int nb = 0; nb < NB32; nb++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int n = n0 + nb * 32 + q * 8 + kg * 4;
+                    if (n < N) {
+                        if (ws) {
+                            // partial sums keep the register layout (split, tile, wave, register group,
+                            // lane): every store is 1 KiB contiguous; the reduction kernel undoes it
+                            const f32x4 o = {acc[mb][nb][q * 4], acc[mb][nb][q * 4 + 1], acc[mb][nb][q * 4 + 2],
+                                             acc[mb][nb][q * 4 + 3]};
+                            // dense: tiles in row-major order; grouped: in the order of the launch
+                            const int64_t tile_id = GROUPED ? (int64_t)blockIdx.x : (int64_t)(m0 / GM) * ((N + GN - 1) / GN) + tile_n;
+                            const int64_t n_tiles_all = GROUPED ? (int64_t)gridDim.x : (int64_t)((M + GM - 1) / GM) * ((N + GN - 1) / GN);
+                            const int64_t slot = (((int64_t)blockIdx.y * n_tiles_all + tile_id) * 4 + wave) * (MB32 * NB32 * 4) +
+                                                 (mb * NB32 + nb) * 4 + q;
+                            *(f32x4 *)(ws + (slot * 64 + lane) * 4) = o;
+                        } else {
+                            typedef AT at4 __attribute__((ext_vector_type(4)));
+                            at4 o;
+#pragma unroll
+                            for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
+                            *(at4 *)(y + (int64_t)m * N + n) = o;
+                        }
+                    }
+                }
+                // one 32x32 block at a time: moving all 128 accumulators to vector registers at
+                // once would set the register footprint of the whole kernel
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    };
+
+    if constexpr (DMA) {
+        // One K step ahead: while step kt is computed the x block of step kt+1 streams into the
+        // other LDS buffer and its weight tiles into the second register set.  The waits this
+        // leaves exposed are covered by the second workgroup that the smaller register footprint
+        // lets a CU hold.
+        auto run = [&](auto mbc) __attribute__((always_inline)) {
+            WRegs w0, w1;
+            constexpr int MBC = decltype(mbc)::value;
+            if constexpr (GTALL) {
+                // Each variant of the main loop derives its addresses from values that are new to the compiler
+                // here: otherwise it computes the scalar addresses of all variants ahead of the branch that
+                // picks one, runs out of scalar registers and spills them (through vector registers to memory).
+                uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)xtile_base);
+                uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(xtile_base >> 32));
+                asm volatile("" : "+s"(lo), "+s"(hi));
+                xtile_base = (uint64_t)lo | ((uint64_t)hi << 32);
+                asm volatile("" : "+v"(wt[0]), "+v"(wt[1]));
+            }
+            const uint32_t voff_tail[2] = {tail_offset(2 * (MBC - 1)), tail_offset(2 * (MBC - 1) + 1)};
+            dma_x(0, xs0, mbc, voff_tail);
+            load_w(0, w0);
+            wait_all_loads();
+            __syncthreads();
+            for (int kt = 0; kt + 1 < Gs; kt += 2) {
+                compute(acc, xs0, w0, mbc, [&](const int point, const int points) __attribute__((always_inline)) {
+                    fetch_units(kt + 1, xs1, w1, point, points, mbc, voff_tail);
+                });
+                wait_all_loads();
+                __syncthreads();
+                compute(acc, xs1, w1, mbc, [&](const int point, const int points) __attribute__((always_inline)) {   // past the end: clamped, unused re-reads
+                    fetch_units(kt + 2, xs0, w0, point, points, mbc, voff_tail);
+                });
+                wait_all_loads();
+                __syncthreads();
+            }
+            if (Gs & 1) compute(acc, xs0, w0, mbc, nothing);
+            epilogue(acc, mbc);
+        };
+        // tail tiles and small expert groups: 32-row blocks without rows of x skip their MFMAs
+        const int mb_cnt = (M - m0 + 31) / 32;
+        if constexpr (MB32 == 8 && !GROUPED) {
+            // the dense launcher hands the tall form whole 256-row tiles only
+            run(full_t());
+        } else if constexpr (MB32 == 8) {
+            // one variant per count: only the last block of a variant may then hold rows past the group's end,
+            // which is what the clamped offsets of its two pieces per wave cover
+            switch (mb_cnt) {
+            case 1: run(std::integral_constant<int, 1>()); break;
+            case 2: run(std::integral_constant<int, 2>()); break;
+            case 3: run(std::integral_constant<int, 3>()); break;
+            case 4: run(std::integral_constant<int, 4>()); break;
+            case 5: run(std::integral_constant<int, 5>()); break;
+            case 6: run(std::integral_constant<int, 6>()); break;
+            case 7: run(std::integral_constant<int, 7>()); break;
+            default: run(full_t()); break;
+            }
+        } else if (mb_cnt <= 1) {
+            run(std::integral_constant<int, 1>());
+        } else if (mb_cnt <= 2) {
+            run(std::integral_constant<int, 2>());
+        } else {
+            run(full_t());
+        }
+    } else {
+    // Software pipeline, two K steps deep: while step kt is computed, the data of step kt+1 is
+    // already in registers (it moves to LDS at the end of step kt) and the loads of step kt+2
+    // are issued.  x rotates through two register sets, the weight tiles through three, hence
+    // the period of six.
+    u32x4 xa[8], xb[8];
+    WRegs w0, w1, w2;
+    load_x(0, xa);
+    load_w(0, w0);
+    load_x(1, xb);
+    load_w(1, w1);
+    store_x(xs0, xa);
+    __syncthreads();
+
+#define LOWBIT_GEMM_STEP(i, cur, nxt, xst, xld, wc, wl)                        \
+    if (kt + (i) < Gs) {                                                       \
+        compute(acc, cur, wc, full_t(), [&](const int point, const int points) __attribute__((always_inline)) { \
+            if (point % MB32 == MB32 - 1) {                                    \
+                const int ks = point / MB32;                                   \
+                if (ks < 2) load_w_nb(kt + (i) + 2, wl, ks);                   \
+                load_x_one(kt + (i) + 2, xld, ks);                             \
+            }                                                                  \
+        });                                                                    \
+        store_x(nxt, xst);                                                     \
+        __syncthreads();                                                       \
+    }
+    for (int kt = 0; kt < Gs; kt += 6) {
+        LOWBIT_GEMM_STEP(0, xs0, xs1, xb, xa, w0, w2)
+        LOWBIT_GEMM_STEP(1, xs1, xs0, xa, xb, w1, w0)
+        LOWBIT_GEMM_STEP(2, xs0, xs1, xb, xa, w2, w1)
+        LOWBIT_GEMM_STEP(3, xs1, xs0, xa, xb, w0, w2)
+        LOWBIT_GEMM_STEP(4, xs0, xs1, xb, xa, w1, w0)
+        LOWBIT_GEMM_STEP(5, xs1, xs0, xa, xb, w2, w1)
+    }
+#undef LOWBIT_GEMM_STEP
+    epilogue(acc, full_t());
+    }
+}
+
+
+}  // namespace lowbit

@@ -275,6 +275,32 @@ def lowbit_grouped_forward(x, w_ptrs, y, group_offsets, n_groups, total_rows, qt
                                        n, k, stream), "lowbit_grouped_forward")
 
 
+_lib.lowbit_grouped_workspace_bytes.argtypes = [c_int, c_int64, c_int64, c_int64]
+_lib.lowbit_grouped_workspace_bytes.restype = c_size_t
+_lib.lowbit_grouped_forward_ws.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int,
+                                           c_int64, c_int64, c_void_p, c_size_t, c_void_p]
+_lib.lowbit_grouped_forward_ws.restype = c_int
+_lib.lowbit_grouped_mlp_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int,
+                                            c_int, c_int64, c_int64, c_int, c_void_p]
+_lib.lowbit_grouped_mlp_forward.restype = c_int
+
+
+def lowbit_grouped_workspace_bytes(n_groups, total_rows, n, k):
+    return int(_lib.lowbit_grouped_workspace_bytes(n_groups, total_rows, n, k))
+
+
+def lowbit_grouped_forward_ws(x, w_ptrs, y, group_offsets, n_groups, total_rows, qtype, act_dtype, n, k, workspace,
+                              workspace_bytes, stream):
+    _check(_lib.lowbit_grouped_forward_ws(x, w_ptrs, y, group_offsets, n_groups, total_rows, qtype, act_dtype,
+                                          n, k, workspace, workspace_bytes, stream), "lowbit_grouped_forward_ws")
+
+
+def lowbit_grouped_mlp_forward(x, gate_ptrs, up_ptrs, y, group_offsets, n_groups, total_rows, qtype, act_dtype, n, k,
+                               act, stream):
+    _check(_lib.lowbit_grouped_mlp_forward(x, gate_ptrs, up_ptrs, y, group_offsets, n_groups, total_rows, qtype,
+                                           act_dtype, n, k, act, stream), "lowbit_grouped_mlp_forward")
+
+
 _lib.lowbit_dequantize_rows.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int64, c_int, c_int,
                                         c_void_p]
 _lib.lowbit_dequantize_rows.restype = c_int

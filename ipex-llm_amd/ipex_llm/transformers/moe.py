@@ -4,8 +4,8 @@ The reference has no fused path for a Mixtral-style block at prefill: the Huggin
 loops over the experts and calls each expert's (converted) LowBitLinear on the rows routed to
 it, then index_adds the weighted result (the same pattern as the reference's own
 transformers/models/qwen2_moe.py:375-430).  `moe_ffn_reference` is that loop;
-`moe_ffn_grouped` computes the same thing with three grouped launches (gate, up, down) over the
-rows sorted by expert.
+`moe_ffn_grouped` computes the same thing with two grouped launches over the rows sorted by expert:
+the fused gate/up projection with the activation in its epilogue, then the down projection.
 """
 import ctypes
 
@@ -55,22 +55,49 @@ class ExpertWeights:
                               "an expert weight was moved or replaced after ExpertWeights was built; build it again")
 
 
-def grouped_forward(x_sorted: torch.Tensor, group_offsets: torch.Tensor, experts: ExpertWeights):
-    """y[r] = x_sorted[r] @ dequant(W[e])^T for group_offsets[e] <= r < group_offsets[e+1]."""
+def _check_grouped(x_sorted, group_offsets, experts):
     invalidInputError(x_sorted.dim() == 2 and x_sorted.shape[1] == experts.in_len and x_sorted.dtype in _DT
                       and x_sorted.dtype != torch.float32, "x must be [rows, K] in fp16 / bf16")
     invalidInputError(group_offsets.dtype == torch.int32 and group_offsets.numel() == len(experts.blobs) + 1
                       and group_offsets.device == x_sorted.device, "group_offsets must be int32 [E + 1] on the GPU")
     experts.check(x_sorted.device)
+
+
+def grouped_forward(x_sorted: torch.Tensor, group_offsets: torch.Tensor, experts: ExpertWeights):
+    """y[r] = x_sorted[r] @ dequant(W[e])^T for group_offsets[e] <= r < group_offsets[e+1]."""
+    _check_grouped(x_sorted, group_offsets, experts)
     x_sorted = x_sorted.contiguous()
     rows = x_sorted.shape[0]
     y = torch.empty((rows, experts.out_len), dtype=x_sorted.dtype, device=x_sorted.device)
     if rows:
+        n_exp = len(experts.blobs)
+        ws_bytes = ggml.lowbit_grouped_workspace_bytes(n_exp, rows, experts.out_len, experts.in_len)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=x_sorted.device)
         with torch.cuda.device(x_sorted.device):
-            ggml.lowbit_grouped_forward(x_sorted.data_ptr(), experts.ptrs.data_ptr(), y.data_ptr(),
-                                        group_offsets.data_ptr(), len(experts.blobs), rows, experts.qtype,
-                                        _DT[x_sorted.dtype], experts.out_len, experts.in_len, _stream())
+            ggml.lowbit_grouped_forward_ws(x_sorted.data_ptr(), experts.ptrs.data_ptr(), y.data_ptr(),
+                                           group_offsets.data_ptr(), n_exp, rows, experts.qtype, _DT[x_sorted.dtype],
+                                           experts.out_len, experts.in_len, ws.data_ptr(), ws_bytes, _stream())
     return y
+
+
+def grouped_mlp_forward(x_sorted: torch.Tensor, group_offsets: torch.Tensor, gates: ExpertWeights,
+                        ups: ExpertWeights, act: int = 0):
+    """h[r] = act(x_sorted[r] @ Wg[e]^T) * (x_sorted[r] @ Wu[e]^T) for the rows of group e, in one launch
+    (act: 0 = SiLU, 1 = tanh-GELU, as in mlp_forward_xpu)."""
+    _check_grouped(x_sorted, group_offsets, gates)
+    invalidInputError((ups.qtype, ups.out_len, ups.in_len) == (gates.qtype, gates.out_len, gates.in_len)
+                      and len(ups.blobs) == len(gates.blobs), "gate and up experts do not fit together")
+    ups.check(x_sorted.device)
+    x_sorted = x_sorted.contiguous()
+    rows = x_sorted.shape[0]
+    h = torch.empty((rows, gates.out_len), dtype=x_sorted.dtype, device=x_sorted.device)
+    if rows:
+        with torch.cuda.device(x_sorted.device):
+            ggml.lowbit_grouped_mlp_forward(x_sorted.data_ptr(), gates.ptrs.data_ptr(), ups.ptrs.data_ptr(),
+                                            h.data_ptr(), group_offsets.data_ptr(), len(gates.blobs), rows,
+                                            gates.qtype, _DT[x_sorted.dtype], gates.out_len, gates.in_len, act,
+                                            _stream())
+    return h
 
 
 def moe_forward_vec(x: torch.Tensor, topk_ids: torch.Tensor, topk_weight: torch.Tensor, gates: ExpertWeights,
@@ -115,7 +142,7 @@ def moe_ffn_reference(hidden, router_logits, w1, w3, w2, top_k=2):
 
 
 def moe_ffn_grouped(hidden, router_logits, g1: ExpertWeights, g3: ExpertWeights, g2: ExpertWeights, top_k=2):
-    """Same result with three grouped launches over the (token, expert) pairs sorted by expert."""
+    """Same result with two grouped launches over the (token, expert) pairs sorted by expert."""
     n_exp = len(g1.blobs)
     weights, experts = route_top_k(router_logits, top_k)
     flat_e = experts.reshape(-1)
@@ -125,7 +152,7 @@ def moe_ffn_grouped(hidden, router_logits, g1: ExpertWeights, g3: ExpertWeights,
     offsets = torch.zeros(n_exp + 1, dtype=torch.int32, device=hidden.device)
     offsets[1:] = torch.cumsum(counts, 0).to(torch.int32)
     xs = hidden[tok]
-    h = F.silu(grouped_forward(xs, offsets, g1)) * grouped_forward(xs, offsets, g3)
+    h = grouped_mlp_forward(xs, offsets, g1, g3)
     y = grouped_forward(h, offsets, g2) * weights.reshape(-1)[order].unsqueeze(-1).to(hidden.dtype)
     out = torch.zeros_like(hidden)
     out.index_add_(0, tok, y)

@@ -123,8 +123,10 @@ def test_llama3_70b_linears(qtype, n, k):
     _linear_case(9300 + qtype + n // 100 + k, qtype, n, k, (1, 16, 1024), torch.bfloat16, 0.015, False)
 
 
-# configs[4]: Mixtral-8x7B expert FFN, fp8_e4m3, 8 experts, 512 tokens, top-2, bf16: the three grouped
-# launches at full size; every expert's sampled rows against the oracle on rows of x routed to it
+# configs[4]: Mixtral-8x7B expert FFN, fp8_e4m3, 8 experts, 512 tokens, top-2, bf16, at full size as
+# moe_ffn_grouped runs it: the fused gate/up launch (SiLU in its epilogue), then the down projection with the
+# K-split workspace; the gate and up products also as plain grouped launches.  Every expert's sampled rows
+# against the oracle on rows of x routed to it.
 def test_mixtral_expert_ffn_full_size():
     n_exp, hid, ffn, tokens, top_k = 8, 4096, 14336, 512, 2
     dtype = torch.bfloat16
@@ -142,7 +144,7 @@ def test_mixtral_expert_ffn_full_size():
     rows_total = tokens * top_k
     xs = hidden[torch.div(order, top_k, rounding_mode="floor")].contiguous()
 
-    def grouped(x, n, k, seed):
+    def experts_of(n, k, seed):
         blobs, checks = [], []
         for e in range(n_exp):
             w = _gpu_weight(seed + e, n, k, 0.02, False)
@@ -152,20 +154,62 @@ def test_mixtral_expert_ffn_full_size():
             blobs.append(blob)
             del w, flat
         ptrs = torch.tensor([b.data_ptr() for b in blobs], dtype=torch.int64, device="cuda")
+        return blobs, ptrs, checks
+
+    def m_sample(seed, e):
+        r0, r1 = int(offs[e]), int(offs[e + 1])
+        return r0 + _sample(seed + 200 + e, r1 - r0, 8) if r1 > r0 else None
+
+    def plain(x, ptrs, checks, n, k, seed, with_workspace):
         y = torch.full((rows_total, n), float("nan"), dtype=dtype, device="cuda")
-        ggml.lowbit_grouped_forward(x.data_ptr(), ptrs.data_ptr(), y.data_ptr(), offsets.data_ptr(), n_exp, rows_total,
-                                    FP8, DT[dtype], n, k, stream())
+        if with_workspace:
+            ws_bytes = ggml.lowbit_grouped_workspace_bytes(n_exp, rows_total, n, k)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+            ggml.lowbit_grouped_forward_ws(x.data_ptr(), ptrs.data_ptr(), y.data_ptr(), offsets.data_ptr(), n_exp,
+                                           rows_total, FP8, DT[dtype], n, k, ws.data_ptr(), ws_bytes, stream())
+        else:
+            ggml.lowbit_grouped_forward(x.data_ptr(), ptrs.data_ptr(), y.data_ptr(), offsets.data_ptr(), n_exp,
+                                        rows_total, FP8, DT[dtype], n, k, stream())
         torch.cuda.synchronize()
         assert not torch.isnan(y).any()
         for e, (rows, blob_rows) in enumerate(checks):
-            r0, r1 = int(offs[e]), int(offs[e + 1])
-            if r1 > r0:
-                m_rows = r0 + _sample(seed + 200 + e, r1 - r0, 8)
-                _check(y, x, blob_rows, FP8, rows, m_rows, k, dtype, ("expert", e, n, k))
+            m_rows = m_sample(seed, e)
+            if m_rows is not None:
+                _check(y, x, blob_rows, FP8, rows, m_rows, k, dtype, ("expert", e, n, k, with_workspace))
         return y
 
-    h1 = grouped(xs, ffn, hid, 9410)                           # w1 (gate)
-    h3 = grouped(xs, ffn, hid, 9430)                           # w3 (up)
-    h = (torch.nn.functional.silu(h1.float()) * h3.float()).to(dtype)
-    del h1, h3
-    grouped(h, hid, ffn, 9450)                                 # w2 (down), K = 14336
+    b1, p1, c1 = experts_of(ffn, hid, 9410)                    # w1 (gate)
+    # w3 (up): the same sampled rows as w1, so that the fused output can be checked entry by entry
+    b3, c3 = [], []
+    for e in range(n_exp):
+        w = _gpu_weight(9430 + e, ffn, hid, 0.02, False)
+        blob, flat = _quantize_full(w, FP8)
+        c3.append((c1[e][0], _oracle_rows(w, flat, FP8, c1[e][0])))
+        b3.append(blob)
+        del w, flat
+    p3 = torch.tensor([b.data_ptr() for b in b3], dtype=torch.int64, device="cuda")
+    plain(xs, p1, c1, ffn, hid, 9410, False)
+    plain(xs, p3, c3, ffn, hid, 9430, False)
+
+    h = torch.full((rows_total, ffn), float("nan"), dtype=dtype, device="cuda")
+    ggml.lowbit_grouped_mlp_forward(xs.data_ptr(), p1.data_ptr(), p3.data_ptr(), h.data_ptr(), offsets.data_ptr(), n_exp,
+                                    rows_total, FP8, DT[dtype], ffn, hid, 0, stream())
+    torch.cuda.synchronize()
+    assert not torch.isnan(h).any()
+    for e in range(n_exp):
+        m_rows = m_sample(9410, e)
+        if m_rows is None:
+            continue
+        rows = c1[e][0]
+        xf = xs[torch.from_numpy(m_rows).cuda()].float().cpu().numpy()
+        gate = orc.mul_mat_exact(c1[e][1], xf, (len(rows), hid), FP8)
+        up = orc.mul_mat_exact(c3[e][1], xf, (len(rows), hid), FP8)
+        want = gate / (1.0 + np.exp(-gate)) * up
+        got = h[torch.from_numpy(m_rows).cuda()][:, torch.from_numpy(rows).cuda()].float().cpu().numpy()
+        assert np.abs(got - want).max() <= 8e-3 * np.abs(want).max(), ("fused gate/up, expert", e)
+    del b1, b3
+
+    b2, p2, c2 = experts_of(hid, ffn, 9450)                    # w2 (down), K = 14336
+    assert ggml.lowbit_grouped_workspace_bytes(n_exp, rows_total, hid, ffn) > 0      # this shape splits K
+    plain(h, p2, c2, hid, ffn, 9450, True)
+    plain(h, p2, c2, hid, ffn, 9450, False)

@@ -1,0 +1,51 @@
+"""The MFMA GEMM kernels keep their MFMAs in inline assembly, which hides from the compiler that accumulator
+blocks are still in flight after them.  ipex-llm_amd/csrc/check_gemm_asm.py looks through the generated assembly
+for what that can break (accumulator blocks copied or read too early, scratch memory, function calls, scalar
+base addresses written by the vector unit right ahead of an LDS-DMA).  Here it runs on one translation unit,
+compiled for gfx950 on the CPU (about a minute); LOWBIT_ASM_CHECK_ALL=1 checks every GEMM translation unit."""
+import glob
+import os
+import subprocess
+import sys
+
+import pytest
+
+CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ipex-llm_amd", "csrc")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+         "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-fast-math", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-S", "--cuda-device-only"]
+
+
+def _units():
+    if os.environ.get("LOWBIT_ASM_CHECK_ALL") == "1":
+        return [os.path.basename(p) for p in sorted(glob.glob(os.path.join(CSRC, "gemm_grouped_*.hip")))] + ["gemm.hip"]
+    return ["gemm_grouped_fp8_e4m3.hip"]
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
+@pytest.mark.parametrize("unit", _units())
+def test_generated_assembly_respects_the_mfma_hazards(unit, tmp_path):
+    listing = str(tmp_path / (unit + ".s"))
+    subprocess.check_call([HIPCC] + FLAGS + ["-c", os.path.join(CSRC, unit), "-o", listing], cwd=CSRC,
+                          stderr=subprocess.DEVNULL)
+    # the 128-row DMA form is held to 128 vector registers, for two workgroups per compute unit, and spills a few
+    out = subprocess.run([sys.executable, os.path.join(CSRC, "check_gemm_asm.py"), listing, "--allow-scratch", "Lb1ELi4E"],
+                         capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout[-4000:]
+    assert out.stdout.count(": ok") >= 3, out.stdout
+
+
+def test_the_checker_sees_a_copy_of_a_fresh_accumulator(tmp_path):
+    bad = tmp_path / "bad.s"
+    bad.write_text("_Z16gemm_mfma_kernelv:\n"
+                   "\tv_accvgpr_write_b32 a0, 0\n"
+                   "\tv_mfma_f32_32x32x16_bf16 a[0:15], v[0:3], v[4:7], a[0:15]\n"
+                   "\tv_mfma_f32_32x32x16_bf16 a[16:31], v[0:3], v[4:7], a[16:31]\n"
+                   "\ts_barrier\n"
+                   "\tv_accvgpr_mov_b32 a40, a0\n"          # written two MFMAs ago: fine
+                   "\tv_accvgpr_mov_b32 a41, a16\n"         # written by the MFMA just issued: not fine
+                   "\ts_endpgm\n")
+    out = subprocess.run([sys.executable, os.path.join(CSRC, "check_gemm_asm.py"), str(bad)], capture_output=True, text=True)
+    assert out.returncode == 1
+    assert "a41, a16" in out.stdout and "a40, a0" not in out.stdout

@@ -7,8 +7,8 @@ import torch
 import lowbit_oracle as orc
 from ipex_llm.ggml.quantize import ggml_tensor_qtype as Q
 from ipex_llm.transformers.low_bit_linear import FP4Params, LowBitLinear
-from ipex_llm.transformers.moe import (ExpertWeights, grouped_forward, moe_ffn_grouped, moe_ffn_reference,
-                                       route_top_k)
+from ipex_llm.transformers.moe import (ExpertWeights, grouped_forward, grouped_mlp_forward, moe_ffn_grouped,
+                                       moe_ffn_reference, route_top_k)
 from gpu_util import weights
 
 pytestmark = pytest.mark.gpu
@@ -46,6 +46,102 @@ def test_grouped_forward_matches_oracle_per_group(qname, dtype):
             tol = 2e-3 if dtype == torch.float16 else 8e-3
             assert np.abs(y[r0:r0 + c] - want).max() <= tol * np.abs(want).max(), (e, c)
         r0 += c
+
+
+# Row counts that put the launch on the 256-row form (more than 96 rows per group on average): a tile for
+# every count of 32-row blocks from 1 to 8, whole tiles, a whole tile plus a short one, an empty group.
+TALL_COUNTS = [257, 0, 1, 33, 65, 97, 129, 161, 193, 225, 256, 300]
+
+
+def _offsets(counts):
+    return torch.tensor(np.concatenate([[0], np.cumsum(counts)]), dtype=torch.int32, device="cuda")
+
+
+@pytest.mark.parametrize("qname,dtype", [("fp8_e4m3", torch.bfloat16), ("sym_int4", torch.float16),
+                                         ("asym_int4", torch.bfloat16), ("nf4", torch.bfloat16),
+                                         ("sym_int8", torch.float16)])
+@pytest.mark.parametrize("k", [384, 2048])
+def test_grouped_forward_tall_form_matches_oracle_per_group(qname, dtype, k):
+    """K = 2048 with 272 columns splits K over the workspace (2 splits of 8 steps), K = 384 does not; both also
+    through the entry point without a workspace."""
+    import ipex_llm.ggml.model.llama.llama_cpp as ggml
+    from gpu_util import DT, stream
+    qtype = Q[qname]
+    n = 272
+    counts = TALL_COUNTS
+    lins, raw = _experts(len(counts), n, k, qtype, 8600)
+    rows = sum(counts)
+    assert (ggml.lowbit_grouped_workspace_bytes(len(counts), rows, n, k) > 0) == (k == 2048)
+    torch.manual_seed(3)
+    x = torch.randn(rows, k).to(dtype).cuda()
+    offs = _offsets(counts)
+    table = ExpertWeights(lins)
+    y_ws = grouped_forward(x, offs, table)
+    y_plain = torch.full((rows + 3, n), float("nan"), dtype=dtype, device="cuda")      # three rows that no group owns
+    ggml.lowbit_grouped_forward(x.data_ptr(), table.ptrs.data_ptr(), y_plain.data_ptr(), offs.data_ptr(), len(counts),
+                                rows, qtype, DT[dtype], n, k, stream())
+    torch.cuda.synchronize()
+    assert torch.isnan(y_plain[rows:]).all() and not torch.isnan(y_plain[:rows]).any()
+    r0 = 0
+    for e, c in enumerate(counts):
+        if c:
+            blob = orc.quantize(raw[e], qtype)
+            want = orc.mul_mat_exact(blob, x[r0:r0 + c].float().cpu().numpy(), (n, k), qtype)
+            tol = 2e-3 if dtype == torch.float16 else 8e-3
+            for got in (y_ws, y_plain):
+                err = np.abs(got[r0:r0 + c].float().cpu().numpy() - want).max()
+                assert err <= tol * np.abs(want).max(), (e, c)
+        r0 += c
+
+
+@pytest.mark.parametrize("qname,dtype,act", [("fp8_e4m3", torch.bfloat16, 0), ("sym_int4", torch.float16, 0),
+                                             ("nf4", torch.bfloat16, 1), ("sym_int8", torch.float16, 1),
+                                             ("asym_int4", torch.float16, 0)])
+@pytest.mark.parametrize("counts", [TALL_COUNTS, [130, 0, 1, 17, 129, 40, 64, 97]])
+def test_grouped_mlp_forward_matches_oracle_per_group(qname, dtype, act, counts):
+    """act(x Wg^T) * (x Wu^T) of every group in one launch; 272 columns = two workgroup tiles and 16 columns."""
+    qtype = Q[qname]
+    n, k = 272, 384
+    gate, raw_g = _experts(len(counts), n, k, qtype, 8700)
+    up, raw_u = _experts(len(counts), n, k, qtype, 8800)
+    rows = sum(counts)
+    torch.manual_seed(4)
+    x = torch.randn(rows, k).to(dtype).cuda()
+    h = grouped_mlp_forward(x, _offsets(counts), ExpertWeights(gate), ExpertWeights(up), act).float().cpu().numpy()
+    r0 = 0
+    for e, c in enumerate(counts):
+        if c:
+            xe = x[r0:r0 + c].float().cpu().numpy()
+            g = orc.mul_mat_exact(orc.quantize(raw_g[e], qtype), xe, (n, k), qtype)
+            u = orc.mul_mat_exact(orc.quantize(raw_u[e], qtype), xe, (n, k), qtype)
+            if act == 0:
+                want = g / (1.0 + np.exp(-g)) * u
+            else:
+                want = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3))) * u
+            tol = 2e-3 if dtype == torch.float16 else 8e-3
+            assert np.abs(h[r0:r0 + c] - want).max() <= tol * np.abs(want).max(), (e, c)
+        r0 += c
+
+
+def test_grouped_entry_points_refuse_bad_arguments():
+    import ipex_llm.ggml.model.llama.llama_cpp as ggml
+    from gpu_util import stream
+    lins, _ = _experts(2, 32, 128, Q["sym_int4"], 8900)
+    table = ExpertWeights(lins)
+    x = torch.zeros(4, 128, dtype=torch.float16, device="cuda")
+    y = torch.zeros(4, 32, dtype=torch.float16, device="cuda")
+    offs = _offsets([2, 2])
+    args = (x.data_ptr(), table.ptrs.data_ptr(), table.ptrs.data_ptr(), y.data_ptr(), offs.data_ptr(), 2, 4,
+            Q["sym_int4"], 0, 32, 128)
+    with pytest.raises(RuntimeError, match="activation"):
+        ggml.lowbit_grouped_mlp_forward(*args, 7, stream())
+    with pytest.raises(RuntimeError, match="null"):
+        ggml.lowbit_grouped_mlp_forward(x.data_ptr(), table.ptrs.data_ptr(), None, y.data_ptr(), offs.data_ptr(), 2, 4,
+                                        Q["sym_int4"], 0, 32, 128, 0, stream())
+    with pytest.raises(RuntimeError, match="f16 or bf16"):
+        ggml.lowbit_grouped_forward_ws(x.data_ptr(), table.ptrs.data_ptr(), y.data_ptr(), offs.data_ptr(), 2, 4,
+                                       Q["sym_int4"], 2, 32, 128, None, 0, stream())
+    assert ggml.lowbit_grouped_workspace_bytes(0, 4, 32, 128) == 0
 
 
 @pytest.mark.parametrize("qname,dtype", [("fp8_e4m3", torch.bfloat16), ("sym_int4", torch.float16)])
