@@ -152,6 +152,12 @@ __device__ inline void wait_all_loads() {
     __builtin_amdgcn_s_waitcnt(0x0F70);
     asm volatile("" ::: "memory");
 }
+// Waits until at most N global loads are outstanding (loads retire in order: the N youngest may stay in flight).
+template <int N> __device__ inline void wait_loads_but() {
+    static_assert(N >= 0 && N < 64, "vmcnt has 6 bits");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+    asm volatile("" ::: "memory");
+}
 
 // The compiler inserts no wait states for an instruction inside inline assembly: a source register
 // written by the VALU instruction just before the MFMA (the packed conversion that ends a

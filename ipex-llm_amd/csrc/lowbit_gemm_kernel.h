@@ -334,6 +334,20 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
         }
     };
 
+    // The same for the deeper pipeline of the grouped tall form (below): the pieces of x of step kt_x first, then the
+    // weight registers of step kt_w, so that the weight loads are the youngest loads in flight when the step ends.
+    auto fetch_units_deep = [&](int kt_x, uint8_t *buf, int kt_w, WRegs &t, const int point, const int points, auto mbc_,
+                                const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
+        constexpr int XU = 2 * decltype(mbc_)::value, UNITS = XU + NB32;
+        const int spread = points * 5 / 8 > 0 ? points * 5 / 8 : 1;
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            if (u < point * UNITS / spread || u >= (point + 1) * UNITS / spread || point >= spread) continue;
+            if (u < XU) dma_x_grouped(kt_x, buf, u, mbc_, voff_tail);
+            else load_w_nb(kt_w, t, u - XU);
+        }
+    };
+
     // One set of accumulators for all variants of the main loop, cleared here.  Every MFMA names its
     // accumulator as an in-out operand of its assembly statement, which keeps each block in the same accumulation
     // registers from here to the epilogue.  It has to: the compiler does not know that the statements are MFMAs
@@ -501,6 +515,41 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
                 asm volatile("" : "+v"(wt[0]), "+v"(wt[1]));
             }
             const uint32_t voff_tail[2] = {tail_offset(2 * (MBC - 1)), tail_offset(2 * (MBC - 1) + 1)};
+            if constexpr (GTALL && MBC < 8) {
+                // Tiles of a few row blocks have short K steps: with one step of prefetch a step lasted as long as
+                // a weight load takes to come back from HBM, whatever it computed (removing the MFMAs of a four-block
+                // tile saved 7 % of its time, removing the weight loads 21 %).  These variants have registers to
+                // spare, so the weights run two steps ahead, through three register sets, and a step ends when
+                // everything but the weight loads it has just issued has landed.  x keeps its two LDS buffers and
+                // one step of prefetch (it comes from L2).  Three weight sets and two buffers: a period of six.
+                constexpr int WLOADS = NB32 * ((F::BITS == 8 ? 2 : 1) * 2 + 1);      // load instructions of load_w_nb, all blocks
+                WRegs w2;
+                dma_x(0, xs0, mbc, voff_tail);
+                load_w(0, w0);
+                load_w(1, w1);
+                wait_all_loads();
+                __syncthreads();
+#define LOWBIT_DEEP_STEP(i, cur, nxt, wc, wl)                                                                  \
+                if (kt + (i) < Gs) {                                                                           \
+                    compute(acc, cur, wc, mbc, [&](const int point, const int points) __attribute__((always_inline)) { \
+                        fetch_units_deep(kt + (i) + 1, nxt, kt + (i) + 2, wl, point, points, mbc, voff_tail); \
+                    });                                                                                        \
+                    wait_loads_but<WLOADS>();                                                                  \
+                    __syncthreads();                                                                           \
+                }
+                for (int kt = 0; kt < Gs; kt += 6) {
+                    LOWBIT_DEEP_STEP(0, xs0, xs1, w0, w2)
+                    LOWBIT_DEEP_STEP(1, xs1, xs0, w1, w0)
+                    LOWBIT_DEEP_STEP(2, xs0, xs1, w2, w1)
+                    LOWBIT_DEEP_STEP(3, xs1, xs0, w0, w2)
+                    LOWBIT_DEEP_STEP(4, xs0, xs1, w1, w0)
+                    LOWBIT_DEEP_STEP(5, xs1, xs0, w2, w1)
+                }
+#undef LOWBIT_DEEP_STEP
+                wait_all_loads();                   // the loads past the end (clamped re-reads) must not outlive the wave's registers
+                epilogue(acc, mbc);
+                return;
+            }
             dma_x(0, xs0, mbc, voff_tail);
             load_w(0, w0);
             wait_all_loads();
