@@ -123,6 +123,45 @@ def test_grouped_mlp_forward_matches_oracle_per_group(qname, dtype, act, counts)
         r0 += c
 
 
+def test_grouped_ffn_replays_correctly_from_a_hip_graph():
+    """The fused gate/up launch and the down projection with its K-split workspace, captured once and replayed
+    with new activations and a new routing (static buffers), with eager work and synchronizations between the
+    replays; every replay must equal the eager result bit for bit."""
+    qtype = Q["fp8_e4m3"]
+    n_exp, hidden, ffn, rows = 6, 256, 2048, 6 * 150
+    w1, _ = _experts(n_exp, ffn, hidden, qtype, 9000)
+    w3, _ = _experts(n_exp, ffn, hidden, qtype, 9100)
+    w2, _ = _experts(n_exp, hidden, ffn, qtype, 9200)
+    g1, g3, g2 = ExpertWeights(w1), ExpertWeights(w3), ExpertWeights(w2)
+    import ipex_llm.ggml.model.llama.llama_cpp as ggml
+    assert ggml.lowbit_grouped_workspace_bytes(n_exp, rows, hidden, ffn) > 0        # the down projection splits K
+    static_x = torch.zeros(rows, hidden, dtype=torch.bfloat16, device="cuda")
+    static_offs = _offsets([150] * n_exp)
+
+    def ffn_of(x, offs):
+        return grouped_forward(grouped_mlp_forward(x, offs, g1, g3), offs, g2)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ffn_of(static_x, static_offs)                      # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = ffn_of(static_x, static_offs)
+    torch.manual_seed(5)
+    for step, counts in enumerate([[150] * 6, [300, 0, 1, 299, 170, 130], [33, 257, 160, 129, 200, 121], [150] * 6]):
+        x = torch.randn(rows, hidden, device="cuda").bfloat16()
+        offs = _offsets(counts)
+        want = ffn_of(x, offs)                             # eager work between the replays
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        static_offs.copy_(offs)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, want), step
+
+
 def test_grouped_entry_points_refuse_bad_arguments():
     import ipex_llm.ggml.model.llama.llama_cpp as ggml
     from gpu_util import stream
