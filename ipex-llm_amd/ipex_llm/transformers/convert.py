@@ -225,6 +225,22 @@ def _replace_with_low_bit_linear(model, qtype, modules_to_not_convert=None,
                 if isinstance(module, nn.Linear):
                     module.weight = None
 
+        elif is_fused_experts(module) and qtype not in (ggml_tensor_qtype["fp16"], ggml_tensor_qtype["bf16"]):
+            # Current transformers keep the experts of a mixture-of-experts block in one module with 3-D
+            # parameters instead of the nn.Linear layers per expert that the reference converts one by one
+            # (convert.py:469-748 on transformers 4.37): the whole module is replaced.
+            from ipex_llm.transformers.low_bit_linear import get_qk_size
+            from ipex_llm.transformers.moe import LowBitExperts
+            _, two_i, hidden = module.gate_up_proj.shape
+            qk = get_qk_size(qtype)
+            if hidden % 64 == 0 and (two_i // 2) % 64 == 0 and (not qk or (hidden % qk == 0 and (two_i // 2) % qk == 0)):
+                model._modules[name] = LowBitExperts.from_fused(module, qtype, convert_shape_only=convert_shape_only,
+                                                                enable_scale_search=enable_scale_search)
+                module.gate_up_proj = None
+                module.down_proj = None
+                has_been_replaced = True
+                continue
+
         elif embedding_qtype is not None and type(module) == nn.Embedding:
             # convert.py:726-729 of the reference
             from ipex_llm.transformers.embedding import LowBitEmbedding
@@ -239,6 +255,15 @@ def _replace_with_low_bit_linear(model, qtype, modules_to_not_convert=None,
                 enable_scale_search=enable_scale_search)
             has_been_replaced = _flag or has_been_replaced
     return model, has_been_replaced
+
+
+def is_fused_experts(module):
+    """A module that holds all experts of a mixture-of-experts block as two 3-D parameters (MixtralExperts and its
+    siblings in current transformers): gate_up_proj [E, 2 I, H], down_proj [E, H, I], and an activation."""
+    gate_up, down = getattr(module, "gate_up_proj", None), getattr(module, "down_proj", None)
+    return (isinstance(gate_up, nn.Parameter) and isinstance(down, nn.Parameter) and gate_up.dim() == 3 and down.dim() == 3
+            and gate_up.shape[0] == down.shape[0] and gate_up.shape[1] == 2 * down.shape[2]
+            and gate_up.shape[2] == down.shape[1] and hasattr(module, "act_fn"))
 
 
 # model types whose attention modules hold q_proj / k_proj / v_proj and get them merged by the reference's

@@ -10,6 +10,7 @@ the fused gate/up projection with the activation in its epilogue, then the down 
 import ctypes
 
 import torch
+import torch.nn as nn
 import torch.nn.functional as F
 
 import ipex_llm.ggml.model.llama.llama_cpp as ggml
@@ -157,3 +158,118 @@ def moe_ffn_grouped(hidden, router_logits, g1: ExpertWeights, g3: ExpertWeights,
     out = torch.zeros_like(hidden)
     out.index_add_(0, tok, y)
     return out
+
+
+def activation_code(act_fn):
+    """0 (SiLU) / 1 (tanh-GELU) for the activations the fused kernels know, None for any other."""
+    name = act_fn.__class__.__name__
+    if isinstance(act_fn, nn.SiLU) or name in ("SiLUActivation", "SiLU"):
+        return 0
+    if (isinstance(act_fn, nn.GELU) and act_fn.approximate == "tanh") or name in ("PytorchGELUTanh", "GELUTanh",
+                                                                               "NewGELUActivation"):
+        return 1
+    return None
+
+
+class LowBitExperts(nn.Module):
+    """The experts of a sparse mixture-of-experts block with low-bit weights.
+
+    With the transformers version the reference pins (4.37) every expert is a small module of three nn.Linear
+    layers, which its `_replace_with_low_bit_linear` turns into LowBitLinear one by one (convert.py:469-748) and
+    the block's Python loop calls in turn.  Current transformers keep all experts of a block in one module with two
+    3-D parameters, `gate_up_proj` [E, 2 I, H] and `down_proj` [E, H, I], and the call
+    `experts(hidden_states [T, H], top_k_index [T, k], top_k_weights [T, k]) -> [T, H]` (MixtralExperts and its
+    siblings).  This module takes that one's place: each expert's three weights become LowBitLinear layers
+    (`gate[e]`, `up[e]`, `down[e]`, so that save_low_bit / load_low_bit carry them like any other), and on the GPU the
+    call runs as two grouped launches over the (token, expert) pairs sorted by expert, or, for one token, as the two
+    launches of `moe_forward_vec`.  Anywhere else it is the per-expert loop over the LowBitLinear layers."""
+
+    def __init__(self, num_experts, hidden_dim, intermediate_dim, qtype, act_fn, enable_scale_search=False):
+        super().__init__()
+        from ipex_llm.transformers.low_bit_linear import LowBitLinear
+        self.num_experts, self.hidden_dim, self.intermediate_dim, self.qtype = num_experts, hidden_dim, intermediate_dim, qtype
+        self.act_fn = act_fn
+
+        def layers(in_f, out_f):
+            return nn.ModuleList([LowBitLinear(in_f, out_f, qtype, bias=False, enable_scale_search=enable_scale_search)
+                                  for _ in range(num_experts)])
+        self.gate, self.up = layers(hidden_dim, intermediate_dim), layers(hidden_dim, intermediate_dim)
+        self.down = layers(intermediate_dim, hidden_dim)
+        self.__dict__["_tables"] = None
+
+    @classmethod
+    def from_fused(cls, module, qtype, convert_shape_only=False, enable_scale_search=False):
+        """From a module that holds `gate_up_proj` [E, 2 I, H], `down_proj` [E, H, I] and `act_fn`."""
+        from ipex_llm.transformers.low_bit_linear import FP4Params
+        gate_up, down = module.gate_up_proj.data, module.down_proj.data
+        n_exp, two_i, hidden = gate_up.shape
+        inter = two_i // 2
+        invalidInputError(tuple(down.shape) == (n_exp, hidden, inter), "gate_up_proj / down_proj shapes do not fit together")
+        new = cls(n_exp, hidden, inter, qtype, module.act_fn, enable_scale_search)
+        device = gate_up.device
+
+        def param(w, in_features):
+            return FP4Params(data=w.contiguous() if w.device.type != "meta" else w, requires_grad=False, quantized=False,
+                             _shape=None, convert_shape_only=convert_shape_only, qtype=qtype, in_features=in_features,
+                             enable_scale_search=enable_scale_search).to(device)
+        for e in range(n_exp):
+            new.gate[e]._parameters["weight"] = param(gate_up[e, :inter], hidden)
+            new.up[e]._parameters["weight"] = param(gate_up[e, inter:], hidden)
+            new.down[e]._parameters["weight"] = param(down[e], inter)
+        if not module.training:
+            new.eval()
+        new.requires_grad_(False)
+        return new
+
+    def _expert_tables(self, device):
+        """Pointer tables of the three projections; built on first use and again when a weight has moved."""
+        tables = self.__dict__["_tables"]
+        if tables is not None:
+            try:
+                for t in tables:
+                    t.check(device)
+                return tables
+            except RuntimeError:
+                pass
+        tables = tuple(ExpertWeights(list(layers)) for layers in (self.gate, self.up, self.down))
+        self.__dict__["_tables"] = tables
+        return tables
+
+    def _grouped_ok(self, x):
+        w = self.gate[0].weight
+        return (x.device.type == "cuda" and x.dtype in (torch.float16, torch.bfloat16) and not self.training
+                and activation_code(self.act_fn) is not None and w.quantized and w.data.device == x.device
+                and ggml.lowbit_tileable(self.qtype, self.intermediate_dim, self.hidden_dim)
+                and ggml.lowbit_tileable(self.qtype, self.hidden_dim, self.intermediate_dim))
+
+    def forward(self, hidden_states, top_k_index, top_k_weights):
+        tokens, top_k = top_k_index.shape
+        if tokens == 0:
+            return torch.zeros_like(hidden_states)
+        if not self._grouped_ok(hidden_states):
+            return self._loop(hidden_states, top_k_index, top_k_weights)
+        act = activation_code(self.act_fn)
+        g1, g3, g2 = self._expert_tables(hidden_states.device)
+        if tokens == 1:
+            return moe_forward_vec(hidden_states, top_k_index, top_k_weights, g1, g3, g2, act)
+        flat_e = top_k_index.reshape(-1)
+        order = torch.argsort(flat_e, stable=True)
+        tok = torch.div(order, top_k, rounding_mode="floor")
+        offsets = torch.zeros(self.num_experts + 1, dtype=torch.int32, device=hidden_states.device)
+        offsets[1:] = torch.cumsum(torch.bincount(flat_e, minlength=self.num_experts)[:self.num_experts], 0).to(torch.int32)
+        h = grouped_mlp_forward(hidden_states[tok], offsets, g1, g3, act)
+        y = grouped_forward(h, offsets, g2) * top_k_weights.reshape(-1)[order].unsqueeze(-1).to(hidden_states.dtype)
+        out = torch.zeros_like(hidden_states)
+        out.index_add_(0, tok, y)
+        return out
+
+    def _loop(self, hidden_states, top_k_index, top_k_weights):
+        out = torch.zeros_like(hidden_states)
+        for e in range(self.num_experts):
+            tok, slot = torch.where(top_k_index == e)
+            if tok.numel() == 0:
+                continue
+            xe = hidden_states[tok]
+            he = self.down[e](self.act_fn(self.gate[e](xe)) * self.up[e](xe))
+            out.index_add_(0, tok, (he * top_k_weights[tok, slot, None]).to(out.dtype))
+        return out

@@ -332,3 +332,41 @@ def test_kernel_choice_boundaries_are_pinned():
         assert ggml.lowbit_forward_plan(qtype, 1, 16, 4096, 4096, True, 1 << 30) == G        # one streaming pass
         assert ggml.lowbit_forward_plan(qtype, 0, 4096, 4096, 4096, True, 1 << 30) == G      # ggml layout: any-shape kernel
     assert ggml.lowbit_forward_plan(99, 1, 1, 64, 128, False) < 0
+
+
+class _FusedExperts(nn.Module):
+    """The shape of MixtralExperts in current transformers: all experts in two 3-D parameters."""
+
+    def __init__(self, n_exp, hidden, inter):
+        super().__init__()
+        self.gate_up_proj = nn.Parameter(torch.empty(n_exp, 2 * inter, hidden))
+        self.down_proj = nn.Parameter(torch.empty(n_exp, hidden, inter))
+        self.act_fn = nn.SiLU()
+
+
+def test_fused_experts_module_is_replaced_expert_by_expert():
+    from ipex_llm.transformers.moe import LowBitExperts
+
+    class Block(nn.Module):
+        def __init__(self, hidden, inter):
+            super().__init__()
+            self.gate = nn.Linear(hidden, 4, bias=False)
+            self.experts = _FusedExperts(4, hidden, inter)
+    with torch.device("meta"):
+        m = nn.Sequential(Block(128, 256)).eval()
+    m, replaced = _replace_with_low_bit_linear(m, Q["sym_int4"], convert_shape_only=True)
+    ex = m[0].experts
+    assert replaced and isinstance(ex, LowBitExperts) and not ex.training
+    assert (ex.num_experts, ex.hidden_dim, ex.intermediate_dim) == (4, 128, 256)
+    for e in range(4):
+        assert tuple(ex.gate[e].weight._shape) == (256, 128) and tuple(ex.up[e].weight._shape) == (256, 128)
+        assert tuple(ex.down[e].weight._shape) == (128, 256) and ex.down[e].weight.quantized
+        assert ex.gate[e].weight.data.numel() == 256 * 128 // 32 * 18 and not ex.gate[e].weight.requires_grad
+    keys = set(m.state_dict().keys())
+    assert {"0.experts.gate.0.weight", "0.experts.up.3.weight", "0.experts.down.2.weight"} <= keys
+    assert not any("gate_up_proj" in k for k in keys)
+    # rows that do not divide into fp8_e4m3's blocks of 128: the module stays as it is
+    with torch.device("meta"):
+        m2 = nn.Sequential(Block(192, 256)).eval()
+    m2, _ = _replace_with_low_bit_linear(m2, Q["fp8_e4m3"], convert_shape_only=True)
+    assert isinstance(m2[0].experts, _FusedExperts)

@@ -227,3 +227,71 @@ def test_moe_forward_vec_equals_the_per_expert_decode_loop(qname, dtype):
     loop = sum(wt * w2[e](torch.nn.functional.silu(w1[e](x)) * w3[e](x)).float()
                for e, wt in zip(ids[0].tolist(), wts[0].tolist())).cpu().numpy()
     assert np.abs(got - loop).max() <= 1e-2 * np.abs(loop).max()
+
+
+def _mixtral_block(n_exp, hidden, inter, top_k, qtype, seed):
+    """A Hugging Face MixtralSparseMoeBlock whose expert weights already are what the oracle dequantizes them to,
+    so that the dense block and its low-bit conversion compute with the same numbers."""
+    transformers = pytest.importorskip("transformers")
+    from transformers.models.mixtral.modeling_mixtral import MixtralSparseMoeBlock
+    cfg = transformers.MixtralConfig(hidden_size=hidden, intermediate_size=inter, num_local_experts=n_exp,
+                                     num_experts_per_tok=top_k, num_hidden_layers=1, num_attention_heads=4,
+                                     num_key_value_heads=4, vocab_size=64)
+    torch.manual_seed(seed)
+    block = MixtralSparseMoeBlock(cfg).eval()
+    with torch.no_grad():
+        for p, shape in ((block.experts.gate_up_proj, (2 * inter, hidden)), (block.experts.down_proj, (hidden, inter))):
+            for e in range(n_exp):
+                w = weights(seed + 10 * e + shape[0], shape)
+                p[e] = torch.from_numpy(orc.dequantize(orc.quantize(w, qtype), qtype, shape))
+        for p in block.gate.parameters():
+            p.copy_(torch.randn_like(p))
+    return block
+
+
+@pytest.mark.parametrize("qname,dtype", [("fp8_e4m3", torch.bfloat16), ("sym_int4", torch.float16)])
+def test_low_bit_experts_take_the_place_of_the_fused_experts_module(qname, dtype):
+    import copy
+    from ipex_llm.transformers.convert import _replace_with_low_bit_linear
+    from ipex_llm.transformers.moe import LowBitExperts
+    qtype = Q[qname]
+    block = _mixtral_block(8, 256, 512, 2, qtype, 9300)
+    dense = copy.deepcopy(block).to(dtype).cuda()
+    low, replaced = _replace_with_low_bit_linear(block, qtype, modules_to_not_convert=["gate"])
+    assert replaced and isinstance(low.experts, LowBitExperts) and isinstance(low.gate, type(dense.gate))
+    low = low.to(dtype).to("cuda")
+    torch.manual_seed(6)
+    for tokens in (300, 1):                                 # grouped launches / the two launches of one decode token
+        x = torch.randn(1, tokens, 256, device="cuda").to(dtype)
+        with torch.no_grad():
+            want = dense(x.clone()).float()
+            got = low(x.clone()).float()
+        assert got.shape == want.shape
+        assert (got - want).abs().max() <= 1e-2 * want.abs().max(), tokens
+
+
+def test_from_pretrained_tiny_mixtral_and_low_bit_round_trip(tmp_path):
+    transformers = pytest.importorskip("transformers")
+    from ipex_llm.transformers import AutoModelForCausalLM
+    from ipex_llm.transformers.moe import LowBitExperts
+    cfg = transformers.MixtralConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2, num_attention_heads=4,
+                                     num_key_value_heads=4, vocab_size=320, max_position_embeddings=64,
+                                     num_local_experts=4, num_experts_per_tok=2)
+    torch.manual_seed(5)
+    hf = transformers.MixtralForCausalLM(cfg).eval()
+    src = tmp_path / "fp"
+    hf.save_pretrained(str(src))
+    model = AutoModelForCausalLM.from_pretrained(str(src), load_in_low_bit="sym_int4", modules_to_not_convert=["lm_head"])
+    experts = [m for m in model.modules() if isinstance(m, LowBitExperts)]
+    assert len(experts) == 2 and experts[0].gate[0].weight.quantized
+    ids = torch.randint(0, 320, (1, 9))
+    with torch.no_grad():
+        want = hf(ids).logits
+        got = model.to("cuda")(ids.cuda()).logits.float().cpu()
+    assert (got - want).abs().mean() / want.abs().mean() < 0.25
+    out = tmp_path / "lowbit"
+    model.save_low_bit(str(out))
+    again = AutoModelForCausalLM.load_low_bit(str(out))
+    with torch.no_grad():
+        got2 = again.to("cuda")(ids.cuda()).logits.float().cpu()
+    assert torch.equal(got, got2)
