@@ -138,7 +138,7 @@ def main(argv):
     bad = 0
     for n, s in enumerate(starts):
         name = text[s].split(":")[0]
-        if "gemm_mfma_kernel" not in name:
+        if "gemm_mfma_kernel" not in name and "gemm_ring_kernel" not in name:
             continue
         e = starts[n + 1] if n + 1 < len(starts) else len(text)
         errors = check_kernel(name, text[s:e], allow, s)

@@ -19,8 +19,9 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
 
 def _units():
     if os.environ.get("LOWBIT_ASM_CHECK_ALL") == "1":
-        return [os.path.basename(p) for p in sorted(glob.glob(os.path.join(CSRC, "gemm_grouped_*.hip")))] + ["gemm.hip"]
-    return ["gemm_grouped_fp8_e4m3.hip"]
+        return ([os.path.basename(p) for p in sorted(glob.glob(os.path.join(CSRC, "gemm_grouped_*.hip")))]
+                + ["gemm.hip", "gemm_ring.hip"])
+    return ["gemm_grouped_fp8_e4m3.hip", "gemm_ring.hip"]
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
