@@ -107,6 +107,15 @@ static int tall_columns(int M, int N, int K, int n_cus) {
     return 2 * left >= 3 * n_cus ? cols : 0;
 }
 
+// Row tiles per band of the kernel's tile order (see the kernel): the row tiles are cut into at most 8 bands, a
+// power of two of them, so that a band of x (band_m * rows per tile * K activations) stays small enough for an
+// XCD's L2 where M allows it.
+static int band_rows(int tiles_m) {
+    int bands = 1;
+    while (bands * 2 <= 8 && bands * 2 <= tiles_m) bands *= 2;
+    return (tiles_m + bands - 1) / bands;
+}
+
 template <int QT, typename AT>
 static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, int K, float *ws, int splits,
                          hipStream_t st) {
@@ -124,23 +133,17 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     const int tall = ws ? 0 : tall_columns(M, N, K, n_cus);
     if (tall > 0) {
         const int tiles_m = M / GM_TALL;
-        int xcd_m = 1;
-        while (xcd_m * 2 <= 8 && xcd_m * 2 <= tiles_m) xcd_m *= 2;
-        const int xcd_n = 8 / xcd_m;
-        const int band_m = (tiles_m + xcd_m - 1) / xcd_m, band_n = (tall + xcd_n - 1) / xcd_n;
-        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL>), dim3(8 * band_m * band_n), dim3(256), 0, st,
-                           (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K, xcd_m, GroupArgs{}, G, (float *)nullptr, 0, tall);
+        const unsigned grid = 8 * (unsigned)(((int64_t)tiles_m * tall + 7) / 8);
+        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL>), dim3(grid), dim3(256), 0, st,
+                           (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K, band_rows(tiles_m), GroupArgs{}, G, (float *)nullptr, 0, tall);
         if (tall == tiles_n_all) return 0;
     }
     const int tn0 = tall, tiles_n = tiles_n_all - tall;
     const int tiles_m = (M + GM - 1) / GM;
-    int xcd_m = 1;                                       // XCDs along M: power of two <= min(8, tiles_m)
-    while (xcd_m * 2 <= 8 && xcd_m * 2 <= tiles_m) xcd_m *= 2;
-    const int xcd_n = 8 / xcd_m;
-    const int band_m = (tiles_m + xcd_m - 1) / xcd_m, band_n = (tiles_n + xcd_n - 1) / xcd_n;
+    const int band_m = band_rows(tiles_m);
     const int k_steps = ws ? (G + splits - 1) / splits : G;
     const int ny = ws ? (G + k_steps - 1) / k_steps : 1;             // splits that actually hold steps
-    dim3 grid(8 * band_m * band_n, ny);
+    dim3 grid(8 * (unsigned)(((int64_t)tiles_m * tiles_n + 7) / 8), ny);
     // Two forms of the kernel.  The DMA form (x straight into LDS, one K step of prefetch, 128
     // vector registers) lets a CU hold two workgroups that cover each other's waits; it wins as
     // soon as there are more workgroups than CUs.  With at most one per CU the register-staged
@@ -148,10 +151,10 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     const bool dma = tiles_m * tiles_n * ny > 256 && M < (1 << 24) && K < (1 << 23);   // 24-bit row offsets
     if (dma)
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
-                           (AT *)y, M, N, K, xcd_m, GroupArgs{}, k_steps, ws, tn0, tiles_n);
+                           (AT *)y, M, N, K, band_m, GroupArgs{}, k_steps, ws, tn0, tiles_n);
     else
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, false, MB32>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
-                           (AT *)y, M, N, K, xcd_m, GroupArgs{}, k_steps, ws, tn0, tiles_n);
+                           (AT *)y, M, N, K, band_m, GroupArgs{}, k_steps, ws, tn0, tiles_n);
     if (ws) {
         const int64_t threads = (int64_t)tiles_m * tiles_n * (GM * GN / 4);
         hipLaunchKernelGGL((splitk_reduce_kernel<AT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, ws,

@@ -110,7 +110,7 @@ __device__ inline float gemm_gate_act(float g, int act) {
 // the epilogue stores act(gate) * up.
 template <int QT, typename AT, bool DMA, int MB, bool GROUPED = false, bool DUAL = false>
 __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
-                                                        AT *__restrict__ y, int M, int N, int K, int xcd_m,
+                                                        AT *__restrict__ y, int M, int N, int K, int band_m,
                                                         const GroupArgs ga, int k_steps,
                                                         float *__restrict__ ws, int tn0, int tn_cnt) {
     using F = Fmt<QT>;
@@ -131,23 +131,27 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
     const int G = K / TILE_COLS;
     const int n_tiles = N / TILE_ROWS;
 
-    // Workgroups are handed to the 8 XCDs round-robin (id % 8) and each XCD has its own L2.  The
-    // output tiles are therefore dealt out so that one XCD owns a block of band_m row-tiles by
-    // band_n column-tiles: its L2 then only has to hold that band of x (re-read by every
-    // column-tile) and sees each weight tile from all its row-tiles at about the same time.
+    // Workgroups are handed to the 8 XCDs round-robin (id % 8) and each XCD has its own L2.  The output tiles
+    // are put in one line - bands of band_m row tiles; within a band column tile by column tile, the band's row
+    // tiles side by side - and each XCD takes an equal eighth of that line (+- one tile): its L2 then holds one
+    // band of x (two where its share crosses a band's end), re-read by every column tile, and sees each weight
+    // tile from all row tiles of the band at about the same time.  Equal shares matter more than whole bands:
+    // with a band per XCD group, 11 row tiles by 43 column tiles put 66 tiles on six XCDs and 44 on two, and 66
+    // tiles are a second round for an XCD whose 32 CUs hold 64 workgroups.
     int m0, tile_n;
     const uint8_t *w_up = nullptr;
     if constexpr (!GROUPED) {
         const int tiles_m = (M + GM - 1) / GM, tiles_n = tn_cnt;
+        const int64_t T = (int64_t)tiles_m * tiles_n;
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-        const int band_m = (tiles_m + xcd_m - 1) / xcd_m;
-        const int xcd_n = 8 / xcd_m;
-        const int band_n = (tiles_n + xcd_n - 1) / xcd_n;
-        const int tile_m = (xcd % xcd_m) * band_m + slot % band_m;
-        tile_n = (xcd / xcd_m) * band_n + slot / band_m;
-        if (slot >= band_m * band_n || tile_m >= tiles_m || tile_n >= tiles_n) return;   // whole workgroup leaves
-        tile_n += tn0;
-        m0 = tile_m * GM;
+        const int first = (int)(T * xcd / 8), count = (int)(T * (xcd + 1) / 8) - first;
+        if (slot >= count) return;                                                   // whole workgroup leaves
+        const int line = first + slot;
+        const int per_band = band_m * tiles_n;
+        const int band = line / per_band, r = line - band * per_band;
+        const int rows_b = tiles_m - band * band_m < band_m ? tiles_m - band * band_m : band_m;   // the last band may be short
+        tile_n = r / rows_b + tn0;
+        m0 = (band * band_m + r % rows_b) * GM;
     } else {
         // every workgroup finds its group by walking the offsets (a handful of scalar loads)
         GroupTile gt;
