@@ -355,3 +355,35 @@ def test_gemm_tall_row_tiles_against_oracle(qtype, dtype, m, n, k):
     y_exact = orc.mul_mat_exact(orc.quantize(w[rows], qtype), x.float().numpy()[ms], (len(rows), k), qtype)
     tol = 2e-3 if dtype == torch.float16 else 8e-3
     assert np.abs(y[np.ix_(ms, rows)] - y_exact).max() <= tol * np.abs(y_exact).max()
+
+
+def test_gemm_tile_line_covers_every_tile_for_any_tile_counts():
+    """The GEMM deals its output tiles to the XCDs in equal shares of one line of tiles; every (row tile, column
+    tile) must be computed exactly once whatever the counts.  Random M / N / K (1 to 13 row tiles, 1 to 12 column
+    tiles, with and without tails; both forms of the kernel, with and without K splits) against the product with
+    the weights the library's own dequantizer returns (the dequantizer is bit-exact against the oracle), on a y
+    that starts as NaN."""
+    rng = np.random.default_rng(77)
+    for case in range(24):
+        qtype = [Q4_0, FP8, Q8_0, NF4][case % 4]
+        dtype = torch.float16 if case % 2 == 0 else torch.bfloat16
+        m = int(rng.integers(17, 1700))
+        n = 16 * int(rng.integers(1, 190))
+        k = 128 * int(rng.integers(1, 7))
+        if case % 5 == 0:
+            m = 128 * int(rng.integers(1, 14))             # whole row tiles
+        w = weights(6000 + case, (n, k))
+        x = acts(6100 + case, m, k, dtype).cuda()
+        blob = dev_quantize(w, qtype, TILED)
+        wd = dev_dequantize(blob, qtype, n, k, TILED, torch.float32)
+        want = x.float() @ wd.t()
+        splits = int(rng.integers(1, 4)) if k >= 512 else 1
+        ws_bytes = max(16, splits * ((m + 127) // 128) * ((n + 255) // 256) * 128 * 1024)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        y = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        ggml.lowbit_gemm_ws(x.data_ptr(), blob.data_ptr(), y.data_ptr(), qtype, TILED, DT[dtype], m, n, k, ws.data_ptr(),
+                            ws_bytes, splits, stream())
+        torch.cuda.synchronize()
+        assert not torch.isnan(y).any(), (case, qtype, m, n, k, splits)
+        tol = 2e-3 if dtype == torch.float16 else 8e-3
+        assert (y.float() - want).abs().max() <= tol * want.abs().max(), (case, qtype, m, n, k, splits)
