@@ -134,8 +134,15 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     if (tall > 0) {
         const int tiles_m = M / GM_TALL;
         const unsigned grid = 8 * (unsigned)(((int64_t)tiles_m * tall + 7) / 8);
-        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL>), dim3(grid), dim3(256), 0, st,
-                           (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K, band_rows(tiles_m), GroupArgs{}, G, (float *)nullptr, 0, tall);
+        // nf4 runs the tall tile with eight waves of 32 columns (two per SIMD cover each other's waits for the code
+        // book reads from LDS: 5-9 % faster than four waves of 64 columns); the other formats are 2-4 % faster
+        // with four waves, which read each x operand from LDS once per two MFMAs.
+        if constexpr (QT == QT_NF4)
+            hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL, false, false, 8>), dim3(grid), dim3(512), 0, st,
+                               (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K, band_rows(tiles_m), GroupArgs{}, G, (float *)nullptr, 0, tall);
+        else
+            hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL>), dim3(grid), dim3(256), 0, st,
+                               (const AT *)x, (const uint8_t *)w, (AT *)y, M, N, K, band_rows(tiles_m), GroupArgs{}, G, (float *)nullptr, 0, tall);
         if (tall == tiles_n_all) return 0;
     }
     const int tn0 = tall, tiles_n = tiles_n_all - tall;

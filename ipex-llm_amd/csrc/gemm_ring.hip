@@ -100,10 +100,13 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
 
     // ---- sources of this lane's share of a stage, for the tile being fetched
     // x: one load moves 8 rows x 128 bytes (64 columns) - whole cache lines - into one 1 KiB piece of
-    // LDS: lane (c, i) = 8*c + i fetches the 16 bytes at row 8*t + i, byte 16*c of the half row h.
-    // Piece q = h * 4*MB + t; wave v fills pieces v*XL .. .  The 16 bytes that lane (kg, r) of the MFMA
-    // wants for 16-column step ks and row r of the tile sit in piece (ks/4) * 4*MB + r/8 at
-    // ((ks%4 * 2 + kg) * 8 + r%8) * 16: eight consecutive lanes read 128 contiguous bytes.
+    // LDS, lane l at byte 16 l of it.  Eight consecutive lanes fetch the eight 16-byte chunks of one row (one
+    // cache line; with the lanes running across rows the loads are 3.6 times slower): lane l = 8*s + c'
+    // fetches row 8*t + (s ^ t%2), chunk c' ^ (s ^ t%2) of the half row h.  Piece q = h * 4*MB + t; wave v
+    // fills pieces v*XL .. .  The 16 bytes that lane (kg, i) of the MFMA wants for 16-column step ks and row i
+    // of a 32-row block sit in piece (ks/4) * 4*MB + 4*mb + i/8 at ((i%8 ^ i/8 % 2) * 8 + ((ks%4 * 2 + kg) ^ i%8)) * 16:
+    // the two xors spread the eight rows of a piece, 128 bytes apart, and the pieces, 1 KiB apart, over the LDS
+    // banks, so that every 16 lanes of a wave-wide read cover all banks once.
     // weights: wave v owns tiles v*TPW .. of the workgroup's NT (tile rows past N are clamped: they are
     // computed and never stored).  Codes: lane l fetches bytes 16l .. of the tile (and of its second
     // KiB for 8-bit codes).  Headers: one 4-byte load per lane, 256 bytes per instruction, which is
@@ -116,9 +119,10 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
 #pragma unroll
         for (int j = 0; j < XL; j++) {
             const int q = wave * XL + j, h = q / (4 * MB), t = q % (4 * MB);
-            int row = tile_m * 32 * MB + t * 8 + (lane & 7);
+            const int r = (lane >> 3) ^ (t & 1);
+            int row = tile_m * 32 * MB + t * 8 + r;
             row = row < M ? row : M - 1;
-            xsrc[j] = (gbytes)x + ((int64_t)row * K + h * 64 + (lane >> 3) * 8) * (int64_t)sizeof(AT);
+            xsrc[j] = (gbytes)x + ((int64_t)row * K + h * 64 + ((lane & 7) ^ r) * 8) * (int64_t)sizeof(AT);
         }
 #pragma unroll
         for (int i = 0; i < TPW; i++) {
@@ -238,8 +242,11 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
                          "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[3][0]), "+a"(acc[3][1]));
     };
     // where the x operand of (16-column step ks, row block mb) starts, and this lane's place in it
-    auto x_piece = [](int ks, int mb) { return ((ks / 4) * 4 * MB + 4 * mb) * 1024 + (ks % 4) * 256; };
-    const int xlane = (i32 >> 3) * 1024 + kg * 128 + (i32 & 7) * 16;
+    auto x_piece = [](int ks, int mb) { return ((ks / 4) * 4 * MB + 4 * mb) * 1024; };
+    int xlane[4];                                    // by ks % 4
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+        xlane[t] = (i32 >> 3) * 1024 + (((i32 & 7) ^ ((i32 >> 3) & 1)) * 8 + ((2 * t + kg) ^ (i32 & 7))) * 16;
     auto compute = [&](const uint8_t *cur, const WRegs &t, bool fetch, int f_slot, int f_kt_now) {
         constexpr int PER = 4 / MB;                  // dequantized pairs per MFMA slot
         V8 xv[2][MB];                                // x operands of this 16-column step and the next
@@ -247,7 +254,7 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
 #pragma unroll
         for (int k = 0; k < 2; k++)
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) xv[k][mb] = *(const V8 *)(cur + xlane + x_piece(k, mb));
+            for (int mb = 0; mb < MB; mb++) xv[k][mb] = *(const V8 *)(cur + xlane[k] + x_piece(k, mb));
 #pragma unroll
         for (int nb = 0; nb < RNB; nb++)
 #pragma unroll
@@ -269,7 +276,7 @@ __global__ __launch_bounds__(64 * RING_WAVES, 1) void gemm_ring_kernel(const AT 
                     }
                 }
                 // two steps ahead: one MFMA slot is shorter than the LDS latency when MB is small
-                if (ks < 6) xv[ks & 1][mb] = *(const V8 *)(cur + xlane + x_piece(ks + 2, mb));
+                if (ks < 6) xv[ks & 1][mb] = *(const V8 *)(cur + xlane[(ks + 2) % 4] + x_piece(ks + 2, mb));
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (ks < 7) {

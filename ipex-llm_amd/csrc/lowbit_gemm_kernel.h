@@ -34,6 +34,8 @@ constexpr int GM_TALL = 256, MB32_TALL = GM_TALL / 32;
 // tall form dequantizes every weight once per 256 rows of x: half the VALU work, half the weight loads and
 // half the barriers per MFMA; its 16 accumulator blocks take all 256 accumulation registers, so a CU holds
 // one workgroup.  tn0 / tn_cnt: the launch covers the column tiles tn0 .. tn0 + tn_cnt - 1 of y.
+// WAVES = 8 (dense tall form only): the same tile with eight waves of 32 weight rows, two per SIMD, 128
+// accumulation registers each; every x operand read from LDS then feeds one MFMA instead of two.
 // Grouped mode (mixture-of-experts): rows offsets[e] .. offsets[e+1]-1 of x use the weight w[e]
 // (and w_up[e] in the fused gate/up form); all pointers are device memory.
 struct GroupArgs {
@@ -108,8 +110,8 @@ __device__ inline float gemm_gate_act(float g, int act) {
 // DUAL (grouped tall form only): the fused gate/up projection of a gated MLP.  The wave's two 32-row weight
 // blocks are the same 32 rows of the gate and of the up weight (a workgroup covers 128 columns of both), and
 // the epilogue stores act(gate) * up.
-template <int QT, typename AT, bool DMA, int MB, bool GROUPED = false, bool DUAL = false>
-__global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
+template <int QT, typename AT, bool DMA, int MB, bool GROUPED = false, bool DUAL = false, int WAVES = 4>
+__global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                         AT *__restrict__ y, int M, int N, int K, int band_m,
                                                         const GroupArgs ga, int k_steps,
                                                         float *__restrict__ ws, int tn0, int tn_cnt) {
@@ -117,7 +119,9 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
     using V8 = typename Vec8<AT>::type;
     static_assert(MB == 4 || (MB == 8 && DMA), "row tiles of 128 rows, or 256 rows in the DMA form");
     static_assert(!DUAL || (GROUPED && MB == 8), "the fused gate/up form exists for grouped launches of the tall form");
+    static_assert(WAVES == 4 || (WAVES == 8 && MB == 8 && DMA && !GROUPED), "eight waves: dense tall form only");
     constexpr int MB32 = MB, GM = 32 * MB;            // shadow the 128-row constants of the file
+    constexpr int NB32 = GN / WAVES / 32;             // 32-row weight blocks per wave: 2, or 1 with eight waves
     // x block of a K step: 8 * MB32 pieces of 1 KiB (layout below), double buffered
     __shared__ __attribute__((aligned(16))) uint8_t xs0[8 * MB32 * 1024];
     __shared__ __attribute__((aligned(16))) uint8_t xs1[8 * MB32 * 1024];
@@ -164,7 +168,7 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
         w = ga.w[group];
         if constexpr (DUAL) w_up = ga.w_up[group];
     }
-    constexpr int GN_WG = DUAL ? GN / 2 : GN, GN_W = DUAL ? GN_WAVE / 2 : GN_WAVE;   // columns of y per workgroup, per wave
+    constexpr int GN_WG = DUAL ? GN / 2 : GN, GN_W = DUAL ? GN_WAVE / 2 : GN / WAVES;   // columns of y per workgroup, per wave
     const int n0 = tile_n * GN_WG + wave * GN_W;
 
     // weight tiles of this lane: block nb covers rows n0 + 32*nb .. +31 (clamped: a tile row past N
@@ -180,36 +184,47 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
     }
 
     // The x block of a K step (128 rows x 256 bytes) sits in LDS as 32 pieces of 1 KiB: piece h * 16 + t
-    // holds rows 8t .. 8t+7 of the half row h (64 columns = 128 bytes), the 16 bytes of (row r, 16-byte
-    // chunk c) at (c * 8 + r % 8) * 16.  Lane (kg, i) of the MFMA reads, for 16-column step ks and row
-    // block mb, piece (ks/4) * 16 + 4*mb + i/8 at ((ks%4 * 2 + kg) * 8 + i%8) * 16: eight consecutive
-    // lanes read 128 contiguous bytes.  The layout is chosen for the DMA form below.
+    // holds rows 8t .. 8t+7 of the half row h (64 columns = 128 bytes = one cache line per row), the 16 bytes
+    // of (row r = 0..7, 16-byte chunk c = 0..7) at ((r ^ t % 2) * 8 + (c ^ r)) * 16.  Two things shape it:
+    //   - One wave-wide load fills one piece with lane l at byte 16 l of it (LDS-DMA writes the lanes to LDS in
+    //     lane order), and eight consecutive lanes fetch the eight chunks of ONE row, a whole cache line: lane
+    //     l = 8 s + c' fetches row r = s ^ t % 2, chunk c' ^ r.  With the lanes running across rows instead
+    //     (lane 8 c + r, eight lines per eight lanes) the same bytes load 3.6 times slower (measured from L2:
+    //     38 against 135 GB/s per CU), and that was a quarter of the GEMM's time.
+    //   - Lane (kg, i) of the MFMA reads, for 16-column step ks and row block mb, row r = i % 8 of piece
+    //     (ks/4) * 16 + 4*mb + i/8 and chunk c = ks%4 * 2 + kg.  Rows lie 128 bytes apart and pieces 1 KiB,
+    //     both a divisor or multiple of the 256 bytes the LDS banks span: the xor with r spreads the eight rows
+    //     of a piece over the banks, the xor with t % 2 puts the next piece's rows on the other half of them,
+    //     so that every 16 lanes cover all banks once (without it a wave-wide 16-byte read runs at half rate:
+    //     303 against 598 GB/s per CU, measured with 8 waves reading back to back).
+    // This lane's row and byte column within an even / odd piece, when it loads one:
+    const int xr_l[2] = {lane >> 3, (lane >> 3) ^ 1};
+    const int xc_l[2] = {(((lane & 7) ^ xr_l[0]) * 16), (((lane & 7) ^ xr_l[1]) * 16)};
     //
-    // Register-staged form: x goes global -> registers -> LDS; a wave-wide load covers 16 rows x 64
-    // bytes: chunk = 4*wave + lane/16 (16 bytes each), row = 16*i + lane%16 for i = 0..7.
-    const int chunk = wave * 4 + (lane >> 4);
+    // Register-staged form: x goes global -> registers -> LDS, piece by piece as above: wave w moves the
+    // pieces 8w .. 8w+7 (half row w/2, rows 64*(w%2) + 8i ..).
     uint32_t xoff[DMA ? 1 : 8];
     int xl[DMA ? 1 : 8];
-    // DMA form: x goes global -> LDS without passing through registers.  One wave-wide instruction
-    // fills one piece: lane 8*c + i fetches the 16 bytes at row 8t + i, byte 16c of the half row - whole
-    // 128-byte lines, 8 per instruction - and the hardware writes the lanes to LDS in lane order.  Wave
-    // w fills pieces 8w .. 8w+7: half row w/2, rows 64*(w%2) + 8j + i.  Rows past M are clamped (the
+    // DMA form: x goes global -> LDS without passing through registers, one instruction per piece.  Wave
+    // w fills pieces 8w .. 8w+7: half row w/2, rows 64*(w%2) + 8j ...  Rows past M are clamped (the
     // offsets are formed with 24-bit multiplies: the launcher keeps M and 2K below 2^24).
-    uint32_t xrow0 = 0, xcol = 0;
+    uint32_t xrow0[2] = {0, 0}, xcol[2] = {0, 0};
     if constexpr (!DMA) {
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const int row_in = i * 16 + r16;
-            int row = m0 + row_in;
+            int row = m0 + 64 * (wave & 1) + 8 * i + xr_l[i & 1];
             row = row < M ? row : M - 1;
-            xoff[i] = (uint32_t)(((int64_t)row * K + chunk * 8) * (int64_t)sizeof(AT));
-            xl[i] = (((chunk >> 3) * (4 * MB32) + (row_in >> 3)) * 64 + (chunk & 7) * 8 + (row_in & 7)) * 16;
+            xoff[i] = (uint32_t)(((int64_t)row * K + (wave >> 1) * 64) * (int64_t)sizeof(AT) + xc_l[i & 1]);
+            xl[i] = (wave * 8 + i) * 1024 + lane * 16;
         }
     } else {
-        xrow0 = m0 + (GM / 2) * (wave & 1) + (lane & 7);
-        xcol = (wave >> 1) * 128 + (lane >> 3) * 16;
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            xrow0[q] = m0 + (GM / 2) * (wave & 1) + xr_l[q];
+            xcol[q] = (wave >> 1) * 128 + xc_l[q];
+        }
     }
-    constexpr int PW = 2 * MB32;                     // pieces of 1 KiB (8 rows of a half row) a wave fetches per K step
+    constexpr int PW = 8 * MB32 / WAVES;                  // pieces of 1 KiB (8 rows of a half row) a wave fetches per K step
     // Split-K: with a workspace the grid has a second dimension, workgroup (t, s) walks the K steps
     // s * k_steps .. and leaves its fp32 partial tile in ws[s]; a second kernel sums the splits.  It
     // fills the machine when the output alone has too few tiles (small M, narrow N).
@@ -227,24 +242,25 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
         const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
         const uint32_t lbase = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + wave * PW * 1024);
-        uint32_t row = xrow0 + 8 * j;
+        uint32_t row = xrow0[j & 1] + 8 * j;
         row = row < (uint32_t)M ? row : (uint32_t)M - 1;
-        const uint8_t *src = xk + (__umul24(row, (uint32_t)K * (uint32_t)sizeof(AT)) + xcol);
+        const uint8_t *src = xk + (__umul24(row, (uint32_t)K * (uint32_t)sizeof(AT)) + xcol[j & 1]);
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                      :: "v"(src), "s"(lbase + j * 1024) : "memory", "m0");
     };
     // Tall form: the per-lane part of the address is a constant 32-bit offset and everything that changes from
     // load to load is scalar arithmetic.  Dense launches hand it whole 256-row tiles only, so no row is clamped.
-    const uint32_t xlane_off = (uint32_t)(lane & 7) * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)(lane >> 3) * 16u;
+    const uint32_t xlane_off = (uint32_t)xr_l[0] * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)xc_l[0];       // even pieces
+    const uint32_t xlane_off_odd = (uint32_t)xr_l[1] * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)xc_l[1];   // odd pieces
     const uint64_t xwave_base = (uint64_t)(uintptr_t)x +
-        ((uint64_t)(m0 + (GM / 2) * (wave & 1)) * (uint64_t)K + (uint64_t)(wave >> 1) * 64u) * sizeof(AT);
+        ((uint64_t)(m0 + (GM / (WAVES / 2)) * (wave % (WAVES / 2))) * (uint64_t)K + (uint64_t)(wave / (WAVES / 2)) * 64u) * sizeof(AT);
     auto dma_x_scalar = [&](int kt, uint8_t *buf, int j) __attribute__((always_inline)) {
         kt = kt0 + (kt < last ? kt : last);
         const uint64_t src = xwave_base + (uint64_t)kt * (TILE_COLS * sizeof(AT)) + (uint64_t)j * 8u * (uint64_t)K * sizeof(AT);
         const uint32_t lbase = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + (wave * PW + j) * 1024);
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"(xlane_off), "s"(src), "s"(lbase) : "memory", "m0");
+                     :: "v"((j & 1) ? xlane_off_odd : xlane_off), "s"(src), "s"(lbase) : "memory", "m0");
     };
     // Grouped tall form: a tile holds rows_here <= 256 rows of its group and only the first MBC 32-row blocks are
     // computed.  Wave w fills the pieces 2j + w % 2 (rows 8 * (2j + w % 2) ..) of half row w / 2 for j < 2 * MBC:
@@ -255,10 +271,11 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
     const int rows_here = __builtin_amdgcn_readfirstlane(M - m0 < GM ? M - m0 : GM);
     uint64_t xtile_base = (uint64_t)(uintptr_t)x + ((uint64_t)m0 * (uint64_t)K + (uint64_t)(wave >> 1) * 64u) * sizeof(AT);
     auto tail_offset = [&](int j) __attribute__((always_inline)) {            // piece j of this wave, rows clamped
-        int row = 8 * (2 * j + (wave & 1)) + (lane & 7);
+        int row = 8 * (2 * j + (wave & 1)) + xr_l[wave & 1];
         row = row < rows_here ? row : rows_here - 1;
-        return (uint32_t)row * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)(lane >> 3) * 16u;
+        return (uint32_t)row * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)xc_l[wave & 1];
     };
+    const uint32_t xlane_off_wave = (wave & 1) ? xlane_off_odd : xlane_off;     // this wave's pieces are all odd or all even
     auto dma_x_grouped = [&](int kt, uint8_t *buf, int j, auto mbc_, const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
         constexpr int MBC = decltype(mbc_)::value;
         kt = kt0 + (kt < last ? kt : last);
@@ -269,7 +286,7 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
         src = uniform64(src);
         const uint32_t lbase = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + ((wave >> 1) * (4 * MB32) + 2 * j + (wave & 1)) * 1024);
-        const uint32_t voff = tail ? voff_tail[j - 2 * (MBC - 1) < 0 ? 0 : j - 2 * (MBC - 1)] : xlane_off;
+        const uint32_t voff = tail ? voff_tail[j - 2 * (MBC - 1) < 0 ? 0 : j - 2 * (MBC - 1)] : xlane_off_wave;
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :: "v"(voff), "s"(src), "s"(lbase) : "memory", "m0");
     };
@@ -342,12 +359,16 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
     // weight registers of step kt_w, so that the weight loads are the youngest loads in flight when the step ends.
     auto fetch_units_deep = [&](int kt_x, uint8_t *buf, int kt_w, WRegs &t, const int point, const int points, auto mbc_,
                                 const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
-        constexpr int XU = 2 * decltype(mbc_)::value, UNITS = XU + NB32;
+        constexpr int XU = GTALL ? 2 * decltype(mbc_)::value : PW, UNITS = XU + NB32;
         const int spread = points * 5 / 8 > 0 ? points * 5 / 8 : 1;
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             if (u < point * UNITS / spread || u >= (point + 1) * UNITS / spread || point >= spread) continue;
-            if (u < XU) dma_x_grouped(kt_x, buf, u, mbc_, voff_tail);
+            if (u < XU) {
+                if constexpr (GTALL) dma_x_grouped(kt_x, buf, u, mbc_, voff_tail);
+                else if constexpr (MB32 == 8) dma_x_scalar(kt_x, buf, u);
+                else dma_x_one(kt_x, buf, u);
+            }
             else load_w_nb(kt_w, t, u - XU);
         }
     };
@@ -382,15 +403,18 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
     // the next step's weights are dequantized after every MFMA, so that LDS latency and the VALU
     // work run in the shadow of the MFMA pipe.  MBC = number of 32-row blocks of x that take part
     // (a compile-time constant: a branch around each MFMA would cut the schedule into pieces).
-    auto x_piece = [](int ks, int mb) __attribute__((always_inline)) { return ((ks / 4) * 4 * MB32 + 4 * mb) * 1024 + (ks % 4) * 256; };
-    const int xlane = (i32 >> 3) * 1024 + kg * 128 + (i32 & 7) * 16;
+    auto x_piece = [](int ks, int mb) __attribute__((always_inline)) { return ((ks / 4) * 4 * MB32 + 4 * mb) * 1024; };
+    int xlane[4];                                     // by ks % 4: the chunk index is xor-ed with the row, not added
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+        xlane[t] = (i32 >> 3) * 1024 + (((i32 & 7) ^ ((i32 >> 3) & 1)) * 8 + ((2 * t + kg) ^ (i32 & 7))) * 16;
     auto compute = [&](auto &acc, const uint8_t *cur, const WRegs &t, auto mbc_, auto &&between) __attribute__((always_inline)) {
         constexpr int MBC = decltype(mbc_)::value;
         constexpr int SLOTS = MBC * NB32, PAIRS = 4 * NB32;   // MFMAs per 16-column step; register pairs to dequantize meanwhile
         V8 xv[MBC];
         u32x4 wv[NB32];
 #pragma unroll
-        for (int mb = 0; mb < MBC; mb++) xv[mb] = *(const V8 *)(cur + xlane + x_piece(0, mb));
+        for (int mb = 0; mb < MBC; mb++) xv[mb] = *(const V8 *)(cur + xlane[0] + x_piece(0, mb));
 #pragma unroll
         for (int nb = 0; nb < NB32; nb++)
 #pragma unroll
@@ -404,16 +428,25 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
                 for (int nb = 0; nb < NB32; nb++) {
                     mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
                     if (ks < 7) {
-                        // pairs [slot * PAIRS / SLOTS, (slot + 1) * PAIRS / SLOTS): spread evenly over the MFMA slots
+                        // pairs [ceil(slot * PAIRS / SLOTS), ceil((slot + 1) * PAIRS / SLOTS)): spread evenly over the
+                        // MFMA slots, the first slot of a row block served first (the second is followed by the LDS
+                        // read and the loads)
                         const int slot_i = mb * NB32 + nb;
 #pragma unroll
                         for (int idx = 0; idx < PAIRS; idx++) {
-                            if (idx < slot_i * PAIRS / SLOTS || idx >= (slot_i + 1) * PAIRS / SLOTS) continue;
+                            if (idx < (slot_i * PAIRS + SLOTS - 1) / SLOTS || idx >= ((slot_i + 1) * PAIRS + SLOTS - 1) / SLOTS) continue;
                             wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);   // (weight block, pair)
                         }
                     }
+                    // An MFMA occupies its pipe for 32 cycles and the wave issues in order: what stands between two
+                    // MFMAs runs in the shadow of the first, and anything beyond 28 cycles of it leaves the pipe idle.
+                    // Left alone the scheduler issues the MFMAs of a row block back to back and everything else after
+                    // them (the second MFMA then waits 32 cycles with nothing to do, and a dozen instructions follow).
+                    // (Not for nf4: its dequantization waits for code book reads from LDS, which the scheduler
+                    // starts earlier when it is free to.)
+                    if (nb + 1 < NB32 && QT != QT_NF4) __builtin_amdgcn_sched_barrier(0);
                 }
-                if (ks < 7) xv[mb] = *(const V8 *)(cur + xlane + x_piece(ks + 1, mb));
+                if (ks < 7) xv[mb] = *(const V8 *)(cur + xlane[(ks + 1) % 4] + x_piece(ks + 1, mb));
                 // keep this order: the scheduler does not know how long an MFMA takes and would
                 // sink the LDS read down to its first use, exposing the LDS latency every time
                 __builtin_amdgcn_sched_barrier(0);
@@ -440,9 +473,14 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
     // before its result may be read; 64 are spent).  The accumulators are operands of the statement,
     // so that no read of them can be scheduled ahead of it.
 #pragma unroll
-    for (int mb = 0; mb < MBC; mb++)
-        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7"
-                     : "+a"(acc[mb][0]), "+a"(acc[mb][1]));
+    for (int mb = 0; mb < MBC; mb++) {
+        if constexpr (NB32 == 2)
+            asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7"
+                         : "+a"(acc[mb][0]), "+a"(acc[mb][1]));
+        else
+            asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7"
+                         : "+a"(acc[mb][0]));
+    }
     // C layout of the 32x32 block: lane = 32*g + col (col = x row within the block), register i =
     // weight row 8*(i/4) + 4*g + i%4: four consecutive n per group of registers
 #pragma unroll
@@ -480,7 +518,7 @@ __global__ __launch_bounds__(256, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kerne
                             // dense: tiles in row-major order; grouped: in the order of the launch
                             const int64_t tile_id = GROUPED ? (int64_t)blockIdx.x : (int64_t)(m0 / GM) * ((N + GN - 1) / GN) + tile_n;
                             const int64_t n_tiles_all = GROUPED ? (int64_t)gridDim.x : (int64_t)((M + GM - 1) / GM) * ((N + GN - 1) / GN);
-                            const int64_t slot = (((int64_t)blockIdx.y * n_tiles_all + tile_id) * 4 + wave) * (MB32 * NB32 * 4) +
+                            const int64_t slot = (((int64_t)blockIdx.y * n_tiles_all + tile_id) * WAVES + wave) * (MB32 * NB32 * 4) +
                                                  (mb * NB32 + nb) * 4 + q;
                             *(f32x4 *)(ws + (slot * 64 + lane) * 4) = o;
                         } else {

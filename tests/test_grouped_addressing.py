@@ -1,8 +1,9 @@
 """Host-side restatement of the index arithmetic of the grouped 256-row GEMM form (lowbit_gemm_kernel.h:
 grouped_tile, dma_x_grouped, the LDS piece layout), checked for what must hold whatever the rows per group:
 every (group, row tile, column tile) is worked on exactly once; every byte the LDS-DMA fetches lies inside x
-(the rows of the last 32-row block are clamped to the group's last row); every LDS piece that the MFMAs of the
-computed blocks read has been filled with the row it stands for."""
+(the rows of the last 32-row block are clamped to the group's last row); every 16-byte operand that the MFMAs of
+the computed blocks read from LDS has been filled with the row and columns it stands for; loads take whole cache
+lines per eight lanes and operand reads spread over all LDS banks."""
 import numpy as np
 import pytest
 
@@ -36,6 +37,21 @@ def grouped_tile(offs, tiles_n, b):
     return None
 
 
+def lane_row_chunk(lane, parity):
+    """Row (0..7) and 16-byte chunk (0..7) of its piece that a lane fetches: eight consecutive lanes take the eight
+    chunks of one row (one cache line), permuted so that the MFMA's reads spread over the LDS banks."""
+    r = (lane >> 3) ^ parity
+    return r, (lane & 7) ^ r
+
+
+def operand_offset(lane, t):
+    """Byte offset, within the four pieces of a 32-row block, of the MFMA operand of `lane` for 16-column step
+    t = ks % 4 of a half row (lowbit_gemm_kernel.h: xlane[t])."""
+    kg, i32 = lane >> 5, lane & 31
+    p, r = i32 >> 3, i32 & 7
+    return p * 1024 + ((r ^ (p & 1)) * 8 + ((2 * t + kg) ^ r)) * 16
+
+
 def check(counts, k, tiles_n=3):
     offs = [0] + [int(v) for v in np.cumsum(counts)]
     total = offs[-1]
@@ -52,32 +68,59 @@ def check(counts, k, tiles_n=3):
         assert offs[e] <= m0 < m_end <= offs[e + 1] and (m0 - offs[e]) % ROWS == 0
         rows_here = min(m_end - m0, ROWS)
         mbc = min((m_end - m0 + 31) // 32, 8)
-        lds = {}
+        lds = {}                                  # 16-byte slot -> (row of the tile, byte column of the K step) it holds
         for wave in range(4):
             h = wave >> 1
             tile_base = (m0 * k + h * 64) * 2
             for j in range(2 * mbc):
                 tail = j >= 2 * (mbc - 1)
                 piece_row = 8 * (2 * j + (wave & 1))
-                for lane in range(64):
-                    if tail:
-                        row = min(piece_row + (lane & 7), rows_here - 1)
-                        src = tile_base + row * k * 2 + (lane >> 3) * 16
-                    else:
-                        row = piece_row + (lane & 7)
-                        src = tile_base + piece_row * k * 2 + (lane & 7) * k * 2 + (lane >> 3) * 16
-                    assert 0 <= src and src + 16 <= x_bytes
-                    assert row == min(piece_row + (lane & 7), rows_here - 1)
-                    assert src - (m0 + row) * k * 2 == h * 128 + (lane >> 3) * 16
                 piece = h * 32 + 2 * j + (wave & 1)
-                assert piece not in lds and piece < 64
-                lds[piece] = piece_row
-        for half in range(2):
+                assert piece < 64
+                for lane in range(64):
+                    r, c = lane_row_chunk(lane, wave & 1)
+                    if tail:
+                        row = min(piece_row + r, rows_here - 1)
+                        src = tile_base + row * k * 2 + c * 16
+                    else:
+                        row = piece_row + r
+                        src = tile_base + piece_row * k * 2 + r * k * 2 + c * 16
+                    assert 0 <= src and src + 16 <= x_bytes
+                    assert row == min(piece_row + r, rows_here - 1)
+                    assert src - (m0 + row) * k * 2 == h * 128 + c * 16
+                    slot = piece * 1024 + lane * 16          # LDS-DMA writes the lanes in lane order
+                    assert slot not in lds
+                    lds[slot] = (row, h * 128 + c * 16)
+        # every operand the MFMAs of the computed blocks read holds the row and columns it stands for
+        for ks in range(8):
             for mb in range(mbc):
-                for q in range(4):
-                    piece = half * 32 + 4 * mb + q
-                    assert lds.get(piece) == 8 * (4 * mb + q)
+                for lane in range(64):
+                    kg, i32 = lane >> 5, lane & 31
+                    slot = ((ks // 4) * 32 + 4 * mb) * 1024 + operand_offset(lane, ks % 4)
+                    want_row = min(32 * mb + i32, rows_here - 1)
+                    assert lds.get(slot) == (want_row, (ks * 16 + kg * 8) * 2), (ks, mb, lane)
     assert len(seen) == sum((c + ROWS - 1) // ROWS for c in counts) * tiles_n
+
+
+def test_operand_reads_cover_all_lds_banks():
+    """A wave-wide 16-byte read is served 16 lanes at a time; the 64 banks are 4 bytes wide.  Each group of 16
+    lanes must touch every bank once, for every 16-column step."""
+    for t in range(4):
+        for g in range(4):
+            banks = []
+            for lane in range(16 * g, 16 * g + 16):
+                o = operand_offset(lane, t)
+                banks += [((o + 4 * i) // 4) % 64 for i in range(4)]
+            assert sorted(banks) == list(range(64)), (t, g)
+
+
+def test_loads_fetch_whole_cache_lines():
+    """Eight consecutive lanes of a load cover one 128-byte line of one row."""
+    for parity in (0, 1):
+        for s8 in range(8):
+            rc = [lane_row_chunk(8 * s8 + i, parity) for i in range(8)]
+            assert len({r for r, _ in rc}) == 1 and sorted(c for _, c in rc) == list(range(8))
+        assert sorted(lane_row_chunk(l, parity)[0] for l in range(0, 64, 8)) == list(range(8))
 
 
 CASES = [[160] * 8, [136, 108, 150, 121, 132, 111, 130, 136], [1, 0, 255, 257, 33, 7, 129, 342], [256] * 8, [0, 0, 5],
