@@ -190,7 +190,9 @@ int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout,
 int lowbit_forward_plan(int qtype, int layout, int64_t M, int64_t N, int64_t K, int have_workspace,
                         size_t workspace_bytes);
 /* The two kernels behind lowbit_forward, for callers (and benchmarks) that choose themselves.
- * waves = 0 lets the library pick the workgroup size of the GEMV. */
+ * waves = 0 lets the library pick the workgroup size of the GEMV.  lowbit_gemm needs y 8-byte aligned
+ * (lowbit_forward sends any other y through the GEMV) and is at its best with y 16-byte aligned: it
+ * then stores whole cache lines. */
 int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
                 int64_t N, int64_t K, int waves, void *stream);
 int lowbit_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,

@@ -189,6 +189,7 @@ static int gemm_entry(const char *what, const void *x, const void *w, void *y, i
     if (int rc = check_mm(what, x, w, y, qtype, layout, act_dtype, M, N, K)) return rc;
     if (M * N == 0) return 0;
     if (K == 0) return fail(LOWBIT_ESHAPE, "%s: K == 0", what);
+    if (((uintptr_t)y) & 7) return fail(LOWBIT_EARG, "%s: y must be 8-byte aligned", what);     // 8-byte stores at the least
     if (workspace && !aligned16(workspace)) return fail(LOWBIT_EARG, "%s: workspace must be 16-byte aligned", what);
     if (splits < 0 || splits > 64) return fail(LOWBIT_EARG, "%s: splits must be 0 (automatic) .. 64", what);
     if (splits > 1) {
@@ -245,7 +246,7 @@ enum { PLAN_GEMV = LOWBIT_PLAN_GEMV, PLAN_RING = LOWBIT_PLAN_RING, PLAN_GEMM = L
 static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, bool have_ws, size_t workspace_bytes,
                         bool y_aligned8, int *splits_out) {
     if (splits_out) *splits_out = 1;
-    if (M <= 16 || layout != LOWBIT_LAYOUT_TILED) return PLAN_GEMV;
+    if (M <= 16 || layout != LOWBIT_LAYOUT_TILED || !y_aligned8) return PLAN_GEMV;            // the MFMA kernels store 8 bytes and more
     if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || K < 128) return PLAN_GEMM;     // reports the error
     const double passes = (double)((M + 15) / 16);
     // a pass cannot be shorter than its workgroups' walk along K (narrow weights leave CUs idle)
@@ -253,13 +254,13 @@ static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, 
     const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
     const int splits = have_ws ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
     const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits);
-    // The ring kernel (y 8-byte aligned) needs the workspace for its partial tiles; given that, it measured
+    // The ring kernel needs the workspace for its partial tiles; given that, it measured
     // faster than or level with the tiled GEMM, split or not, below M = 512 and about 7e10 FLOP (sym_int4 and
     // sym_int8, seven shapes from [1024 x 8192] to [28672 x 8192]).  With nf4, whose code-book lookups weigh
     // on the GEMM's tighter loop, it stays ahead at larger M as well while the GEMM's tiles are no more
     // than one per CU (Llama-3-70B set at M = 512 / 1024: 755 / 808 against 706 / 761 TFLOP/s).  Its own
     // estimate decides against the GEMV.
-    if (y_aligned8 && have_ws && ring_range(qtype, M, N, K) &&
+    if (have_ws && ring_range(qtype, M, N, K) &&
         ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes)
         return ring_time_us((int)M, (int)N, (int)K, qtype, true) < t_gemv ? PLAN_RING : PLAN_GEMV;
     if (t_gemv < t_gemm) return PLAN_GEMV;

@@ -483,11 +483,72 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     }
     // C layout of the 32x32 block: lane = 32*g + col (col = x row within the block), register i =
     // weight row 8*(i/4) + 4*g + i%4: four consecutive n per group of registers
+    //
+    // Straight from these registers a store instruction writes 16 bytes to each of 32 rows of y, 32 partly written
+    // cache lines per instruction, under a row and a column test each.  So each wave first lays its rows out in
+    // LDS - the x buffers, which nobody reads any more - and then stores them with eight (four) consecutive
+    // lanes per row, whole 128 (64) byte runs, eight (sixteen) rows per instruction.  Row r of the wave's part
+    // takes CH 16-byte chunks, chunk c at position c ^ r % CH, which spreads the writes of the 32 rows of a block
+    // over the LDS banks.  Needs y 16-byte aligned; split-K partial sums keep their own layout.
+    constexpr int CH = GN_W * (int)sizeof(AT) / 16;          // 16-byte chunks per row of this wave's columns
+    constexpr int REGION = GM * CH * 16;                     // bytes per wave: WAVES / 2 of them fit an x buffer
+    static_assert(REGION * (WAVES / 2) <= 8 * MB32 * 1024, "a wave's rows fit its share of an x buffer");
+    static_assert(CH == (DUAL ? 4 : NB32 * 4), "one chunk per group of four accumulator registers and kg pair");
+    if (!ws && (((uintptr_t)y) & 15) == 0) {
+        typedef AT at4 __attribute__((ext_vector_type(4)));
+        __syncthreads();                                     // every wave is done with its operand reads
+        uint8_t *const stage = (wave < WAVES / 2 ? xs0 : xs1) + (wave % (WAVES / 2)) * REGION;
+        uint8_t *wpos[CH];                                   // where this lane's 8 bytes of chunk c go, row block 0
+#pragma unroll
+        for (int c = 0; c < CH; c++) wpos[c] = stage + i32 * (CH * 16) + ((c ^ (i32 & (CH - 1))) * 16) + kg * 8;
+#pragma unroll
+        for (int mb = 0; mb < MBC; mb++) {
+#pragma unroll
+            for (int nb = 0; nb < (DUAL ? 1 : NB32); nb++) {
+                // (keeps the block in its accumulation registers up to here: the compiler would otherwise read
+                // all blocks into vector registers ahead of the branch that picks this form of the epilogue)
+                if constexpr (DUAL) asm volatile("" : "+a"(acc[mb][0]), "+a"(acc[mb][1]));
+                else asm volatile("" : "+a"(acc[mb][nb]));
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    at4 o;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        if constexpr (DUAL) o[i] = to_at<AT>(gemm_gate_act(acc[mb][0][q * 4 + i], ga.act) * acc[mb][1][q * 4 + i]);
+                        else o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
+                    }
+                    *(at4 *)(wpos[nb * 4 + q] + mb * 32 * (CH * 16)) = o;
+                }
+                __builtin_amdgcn_sched_barrier(0);           // one 32x32 block at a time (register footprint)
+            }
+        }
+        // the rows were written by other lanes of this wave: LDS serves a wave's accesses in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int RPI = 64 / CH;                         // rows per store instruction
+        const int row_l = lane / CH, cs = lane % CH;
+        const int n = n0 + ((cs ^ (row_l & (CH - 1))) * 8);  // (RPI is a multiple of CH: the same for every j)
+        const int rows_left = n < N ? M - m0 - row_l : 0;    // this lane stores row j * RPI + row_l while that is below
+        AT *const yp = y + (int64_t)(m0 + row_l) * N + n;
+        const uint8_t *const rpos = stage + lane * 16;
+#pragma unroll
+        for (int j0 = 0; j0 < MBC * 32 / RPI; j0 += 8) {
+            u32x4 v[8];
+#pragma unroll
+            for (int j = j0; j < j0 + 8 && j < MBC * 32 / RPI; j++) v[j - j0] = *(const u32x4 *)(rpos + j * 1024);
+#pragma unroll
+            for (int j = j0; j < j0 + 8 && j < MBC * 32 / RPI; j++)
+                if (j * RPI < rows_left) *(u32x4 *)(yp + (int64_t)j * RPI * N) = v[j - j0];
+        }
+        return;
+    }
 #pragma unroll
     for (int mb = 0; mb < MBC; mb++) {
         const int m = m0 + mb * 32 + i32;
         if constexpr (DUAL) {
             // both blocks hold the same 32 columns of y: the gate branch in block 0, the up branch in block 1
+            asm volatile("" : "+a"(acc[mb][0]), "+a"(acc[mb][1]));     // (stay in accumulation registers up to here)
             if (m < M) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
@@ -503,9 +564,11 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-        } else if (m < M) {
+        } else {
 #pragma unroll
             for (int nb = 0; nb < NB32; nb++) {
+                asm volatile("" : "+a"(acc[mb][nb]));                    // (stay in accumulation registers up to here)
+                if (m < M) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const int n = n0 + nb * 32 + q * 8 + kg * 4;
@@ -529,6 +592,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                             *(at4 *)(y + (int64_t)m * N + n) = o;
                         }
                     }
+                }
                 }
                 // one 32x32 block at a time: moving all 128 accumulators to vector registers at
                 // once would set the register footprint of the whole kernel

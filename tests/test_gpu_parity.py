@@ -387,3 +387,28 @@ def test_gemm_tile_line_covers_every_tile_for_any_tile_counts():
         assert not torch.isnan(y).any(), (case, qtype, m, n, k, splits)
         tol = 2e-3 if dtype == torch.float16 else 8e-3
         assert (y.float() - want).abs().max() <= tol * want.abs().max(), (case, qtype, m, n, k, splits)
+
+
+@pytest.mark.gpu
+def test_gemm_output_off_16_byte_alignment_equals_aligned_output():
+    """With y 16-byte aligned the GEMM lays a wave's rows out in LDS and stores whole cache lines; any other y takes
+    the stores straight from the accumulator layout.  Both must give the same bits, tails in M and N included, in
+    both forms of the kernel.  (A y that is not 8-byte aligned is refused.)"""
+    for case, (qtype, dtype, m, n, k) in enumerate([(Q4_0, torch.float16, 200, 528, 256), (NF4, torch.bfloat16, 512, 8192 + 16, 256),
+                                                    (FP8, torch.bfloat16, 2048, 8192, 128), (Q8_0, torch.float16, 77, 48, 384)]):
+        w = weights(6400 + case, (n, k))
+        x = acts(6500 + case, m, k, dtype).cuda()
+        blob = dev_quantize(w, qtype, TILED)
+        y0 = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        ggml.lowbit_gemm(x.data_ptr(), blob.data_ptr(), y0.data_ptr(), qtype, TILED, DT[dtype], m, n, k, stream())
+        for shift in (4,):                                    # 8 bytes off: the least the GEMM entry points accept
+            flat = torch.full((m * n + 8,), float("nan"), dtype=dtype, device="cuda")
+            y1 = flat[shift:shift + m * n].view(m, n)
+            assert y1.data_ptr() % 16 == 2 * shift
+            ggml.lowbit_gemm(x.data_ptr(), blob.data_ptr(), y1.data_ptr(), qtype, TILED, DT[dtype], m, n, k, stream())
+            torch.cuda.synchronize()
+            assert not torch.isnan(y0).any()
+            assert torch.equal(y0, y1), (qtype, m, n, k, shift)
+            assert torch.isnan(flat[:shift]).all() and torch.isnan(flat[shift + m * n:]).all()
+        with pytest.raises(RuntimeError, match="8-byte aligned"):
+            ggml.lowbit_gemm(x.data_ptr(), blob.data_ptr(), y0.data_ptr() + 2, qtype, TILED, DT[dtype], m, n, k, stream())
