@@ -96,7 +96,7 @@ int gemm_splits(int M, int N, int K, size_t ws_bytes) {
 // fill the machine themselves.  Measured on MI355X: a machine full of tall tiles runs 4-7 % (sym_int4) to
 // 10 % (nf4) faster than the 128-row form with two workgroups per CU, which the idle CUs of a thin remainder
 // eat up again ([11008 x 4096] at M = 2048: 32 tall columns + 11 left over, no faster than 688 small tiles).
-static int tall_columns(int M, int N, int K, int n_cus) {
+static int tall_columns(int M, int N, int K, int n_cus, bool heavy_dequant) {
     if (M < 2 * GM_TALL || M % GM_TALL || M >= (1 << 24) || K >= (1 << 23)) return 0;
     const int tiles_m = M / GM_TALL, tiles_n = (N + GN - 1) / GN;
     const int rounds = tiles_m * tiles_n / n_cus;
@@ -104,6 +104,9 @@ static int tall_columns(int M, int N, int K, int n_cus) {
     int cols = rounds * n_cus / tiles_m;
     if (cols >= tiles_n) return tiles_n;
     const int left = (tiles_n - cols) * (M / GM);        // 128-row tiles of the remainder
+    // sym_int8 and nf4 pay most per weight for the dequantization, which the tall form does half as often: for them
+    // it wins with any remainder ([11008 x 4096] at M = 2048: +11 % and +5 %; sym_int4 +1 %, fp8_e4m3 -3 %)
+    if (heavy_dequant) return cols;
     return 2 * left >= 3 * n_cus ? cols : 0;
 }
 
@@ -130,7 +133,7 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     }();
     // tall form on the left columns, 128-row form on the rest (both in the same stream, the second starts when
     // the tall tiles, which all take the same time, are done)
-    const int tall = ws ? 0 : tall_columns(M, N, K, n_cus);
+    const int tall = ws ? 0 : tall_columns(M, N, K, n_cus, QT == QT_SYM_INT8 || QT == QT_NF4);
     if (tall > 0) {
         const int tiles_m = M / GM_TALL;
         const unsigned grid = 8 * (unsigned)(((int64_t)tiles_m * tall + 7) / 8);
@@ -151,11 +154,12 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     const int k_steps = ws ? (G + splits - 1) / splits : G;
     const int ny = ws ? (G + k_steps - 1) / k_steps : 1;             // splits that actually hold steps
     dim3 grid(8 * (unsigned)(((int64_t)tiles_m * tiles_n + 7) / 8), ny);
-    // Two forms of the kernel.  The DMA form (x straight into LDS, one K step of prefetch, 128
-    // vector registers) lets a CU hold two workgroups that cover each other's waits; it wins as
-    // soon as there are more workgroups than CUs.  With at most one per CU the register-staged
-    // form with its deeper prefetch is faster.
-    const bool dma = tiles_m * tiles_n * ny > 256 && M < (1 << 24) && K < (1 << 23);   // 24-bit row offsets
+    // Two forms of the kernel.  The DMA form (x straight into LDS, one K step of prefetch, 128 vector registers)
+    // lets a CU hold two workgroups that cover each other's waits, and is 4-8 % ahead with a single workgroup per
+    // CU as well - except with nf4, whose code book reads compete with the DMA for LDS: there the register-staged
+    // form with its deeper prefetch is 4 % faster while there is at most one workgroup per CU.
+    const bool fits24 = M < (1 << 24) && K < (1 << 23);              // 24-bit row offsets
+    const bool dma = fits24 && (QT != QT_NF4 || tiles_m * tiles_n * ny > 256);
     if (dma)
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
                            (AT *)y, M, N, K, band_m, GroupArgs{}, k_steps, ws, tn0, tiles_n);

@@ -313,9 +313,9 @@ def test_kernel_choice_boundaries_are_pinned():
     ms = (1, 16, 17, 32, 64, 128, 256, 511, 512, 1024, 2048)
     #                         1  16  17  32  64 128 256 511 512 1024 2048
     table = {
-        (2, 4096, 4096):   ([G, G, G, G, R, R, R, R, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
+        (2, 4096, 4096):   ([G, G, G, G, R, R, R, R, R, R, M], [G, G, G, G, G, G, M, M, M, M, M]),
         (2, 11008, 4096):  ([G, G, R, R, R, R, R, R, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
-        (2, 4096, 11008):  ([G, G, R, R, R, R, R, R, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
+        (2, 4096, 11008):  ([G, G, R, R, R, R, R, R, R, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
         (3, 11008, 4096):  ([G, G, R, R, R, R, R, R, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
         (10, 8192, 8192):  ([G, G, R, R, R, R, R, R, R, R, M], [G, G, G, G, G, G, M, M, M, M, M]),
         (10, 1024, 8192):  ([G, G, G, G, R, R, R, R, R, R, R], [G, G, G, G, G, G, G, M, M, M, M]),
