@@ -494,7 +494,32 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     constexpr int REGION = GM * CH * 16;                     // bytes per wave: WAVES / 2 of them fit an x buffer
     static_assert(REGION * (WAVES / 2) <= 8 * MB32 * 1024, "a wave's rows fit its share of an x buffer");
     static_assert(CH == (DUAL ? 4 : NB32 * 4), "one chunk per group of four accumulator registers and kg pair");
-    if (!ws && (((uintptr_t)y) & 15) == 0) {
+    if constexpr (!DUAL) {
+        if (ws) {
+            // Partial sums of a K split keep the register layout (split, tile, wave, register group, lane): every
+            // store is 1 KiB contiguous, straight from the accumulation registers, whole tiles whatever M and N
+            // (the workspace holds whole tiles; the reduction kernel reads what lies inside y and undoes the layout).
+            // dense: tiles in row-major order; grouped: in the order of the launch
+            const int64_t tile_id = GROUPED ? (int64_t)blockIdx.x : (int64_t)(m0 / GM) * ((N + GN - 1) / GN) + tile_n;
+            const int64_t n_tiles_all = GROUPED ? (int64_t)gridDim.x : (int64_t)((M + GM - 1) / GM) * ((N + GN - 1) / GN);
+            float *const wp = ws + ((((int64_t)blockIdx.y * n_tiles_all + tile_id) * WAVES + wave) * (MB32 * NB32 * 4)) * 256 + lane * 4;
+#pragma unroll
+            for (int mb = 0; mb < MBC; mb++) {
+#pragma unroll
+                for (int nb = 0; nb < NB32; nb++) {
+                    asm volatile("" : "+a"(acc[mb][nb]));            // (stay in accumulation registers up to here)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const f32x4 o = {acc[mb][nb][q * 4], acc[mb][nb][q * 4 + 1], acc[mb][nb][q * 4 + 2], acc[mb][nb][q * 4 + 3]};
+                        *(f32x4 *)(wp + ((mb * NB32 + nb) * 4 + q) * 256) = o;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            return;
+        }
+    }
+    if ((((uintptr_t)y) & 15) == 0) {
         typedef AT at4 __attribute__((ext_vector_type(4)));
         __syncthreads();                                     // every wave is done with its operand reads
         uint8_t *const stage = (wave < WAVES / 2 ? xs0 : xs1) + (wave % (WAVES / 2)) * REGION;
@@ -573,24 +598,11 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                 for (int q = 0; q < 4; q++) {
                     const int n = n0 + nb * 32 + q * 8 + kg * 4;
                     if (n < N) {
-                        if (ws) {
-                            // partial sums keep the register layout (split, tile, wave, register group,
-                            // lane): every store is 1 KiB contiguous; the reduction kernel undoes it
-                            const f32x4 o = {acc[mb][nb][q * 4], acc[mb][nb][q * 4 + 1], acc[mb][nb][q * 4 + 2],
-                                             acc[mb][nb][q * 4 + 3]};
-                            // dense: tiles in row-major order; grouped: in the order of the launch
-                            const int64_t tile_id = GROUPED ? (int64_t)blockIdx.x : (int64_t)(m0 / GM) * ((N + GN - 1) / GN) + tile_n;
-                            const int64_t n_tiles_all = GROUPED ? (int64_t)gridDim.x : (int64_t)((M + GM - 1) / GM) * ((N + GN - 1) / GN);
-                            const int64_t slot = (((int64_t)blockIdx.y * n_tiles_all + tile_id) * WAVES + wave) * (MB32 * NB32 * 4) +
-                                                 (mb * NB32 + nb) * 4 + q;
-                            *(f32x4 *)(ws + (slot * 64 + lane) * 4) = o;
-                        } else {
-                            typedef AT at4 __attribute__((ext_vector_type(4)));
-                            at4 o;
+                        typedef AT at4 __attribute__((ext_vector_type(4)));
+                        at4 o;
 #pragma unroll
-                            for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
-                            *(at4 *)(y + (int64_t)m * N + n) = o;
-                        }
+                        for (int i = 0; i < 4; i++) o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
+                        *(at4 *)(y + (int64_t)m * N + n) = o;
                     }
                 }
                 }
