@@ -15,7 +15,9 @@ compiler went along with it, per kernel of an assembly listing (hipcc -S --cuda-
   3. the kernel uses no scratch memory and calls no function (a variant of the main loop that is not inlined
      keeps its closure in scratch and reads the weights with flat loads);
   4. no LDS-DMA takes its scalar base address from a v_readfirstlane less than 5 wait states earlier (VALU
-     write of an SGPR followed by a VMEM read of it).
+     write of an SGPR followed by a VMEM read of it);
+  5. no MFMA reads a vector register as its A or B operand that a VALU instruction wrote less than 2 wait states
+     earlier (the kernels leave the wait states out where the operands are ready long before).
 
 usage: check_gemm_asm.py listing.s [--allow-scratch SUBSTRING ...]
 Exit status 0 when every kernel passes, 1 otherwise.
@@ -49,6 +51,15 @@ def regs(spec):
     if m:
         return set(range(int(m.group(1)), int(m.group(2)) + 1))
     m = re.match(r"a(\d+)$", spec)
+    return {int(m.group(1))} if m else set()
+
+
+def vregs(spec):
+    """'v[4:7]' or 'v5' -> set of register numbers."""
+    m = re.match(r"v\[(\d+):(\d+)\]", spec)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"v(\d+)$", spec)
     return {int(m.group(1))} if m else set()
 
 
@@ -109,6 +120,20 @@ def check_kernel(name, lines, allow_scratch, first_line=0):
         if t.startswith("scratch_") and not any(a in name for a in allow_scratch):
             errors.append(f"line {no + 1}: scratch access: {t}")
             break
+        m = re.match(r"v_mfma_\S+ a\[\d+:\d+\], (v\[\d+:\d+\]), (v\[\d+:\d+\])", t)
+        if m:
+            src = vregs(m.group(1)) | vregs(m.group(2))
+            w = 0
+            for j in range(k - 1, -1, -1):
+                tj = ins[j][1]
+                if tj.startswith("v_") and not tj.startswith("v_mfma"):
+                    mm = re.match(r"\S+ (v\[\d+:\d+\]|v\d+)[, ]", tj + " ")
+                    if mm and (vregs(mm.group(1)) & src):
+                        errors.append(f"line {no + 1}: MFMA operand written by VALU {w} wait states earlier: {tj}")
+                        break
+                w += wait_states(tj)
+                if w >= 2 or re.match(r"s_branch|s_cbranch|s_endpgm|s_setpc_b64", tj):
+                    break
         m = re.match(r"global_load_lds_dwordx4 v\d+, s\[(\d+):(\d+)\]", t)
         if m:
             base = {int(m.group(1)), int(m.group(2))}

@@ -160,13 +160,17 @@ template <int N> __device__ inline void wait_loads_but() {
 }
 
 // The compiler inserts no wait states for an instruction inside inline assembly: a source register
-// written by the VALU instruction just before the MFMA (the packed conversion that ends a
-// dequantization) needs two wait states before the MFMA may read it.
-__device__ inline void mfma_acc(f32x16 &c, f16x8 a, f16x8 b) {
-    asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+// written by a VALU instruction within the two instructions ahead of the MFMA (the packed conversion
+// that ends a dequantization) needs two wait states before the MFMA may read it.  NOP = false is for
+// loops whose operands are ready long before (check_gemm_asm.py verifies that in the generated code):
+// with one wave per SIMD every instruction between two MFMAs is issue time the MFMA has to cover.
+template <bool NOP = true> __device__ inline void mfma_acc(f32x16 &c, f16x8 a, f16x8 b) {
+    if constexpr (NOP) asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    else asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
-__device__ inline void mfma_acc(f32x16 &c, bf16x8 a, bf16x8 b) {
-    asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+template <bool NOP = true> __device__ inline void mfma_acc(f32x16 &c, bf16x8 a, bf16x8 b) {
+    if constexpr (NOP) asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    else asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
 }  // namespace lowbit

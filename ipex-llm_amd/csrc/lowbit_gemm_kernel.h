@@ -419,6 +419,14 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
         for (int nb = 0; nb < NB32; nb++)
 #pragma unroll
             for (int p = 0; p < 4; p++) wv[nb][p] = dequant_pair(t, 0, nb, p);
+        // From here on every operand of an MFMA is written at least a 16-column step ahead of it - except with a
+        // single row block, where the next step's weights are dequantized right behind the MFMA that precedes
+        // their use: those variants keep the two wait states ahead of every MFMA, the others spend them once.
+        constexpr bool WAIT_STATES = MBC * NB32 < 4;
+        if constexpr (!WAIT_STATES) {
+            asm volatile("s_nop 1" : "+v"(wv[0]));
+            if constexpr (NB32 == 2) asm volatile("" : "+v"(wv[1]));
+        }
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
             u32x4 wn[NB32];
@@ -426,7 +434,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
             for (int mb = 0; mb < MBC; mb++) {
 #pragma unroll
                 for (int nb = 0; nb < NB32; nb++) {
-                    mfma_acc(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    mfma_acc<WAIT_STATES>(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
                     if (ks < 7) {
                         // pairs [ceil(slot * PAIRS / SLOTS), ceil((slot + 1) * PAIRS / SLOTS)): spread evenly over the
                         // MFMA slots, the first slot of a row block served first (the second is followed by the LDS

@@ -1,7 +1,8 @@
 """The MFMA GEMM kernels keep their MFMAs in inline assembly, which hides from the compiler that accumulator
 blocks are still in flight after them.  ipex-llm_amd/csrc/check_gemm_asm.py looks through the generated assembly
 for what that can break (accumulator blocks copied or read too early, scratch memory, function calls, scalar
-base addresses written by the vector unit right ahead of an LDS-DMA).  Here it runs on one translation unit,
+base addresses written by the vector unit right ahead of an LDS-DMA, MFMA operands written by the vector unit
+right ahead of the MFMA).  Here it runs on one translation unit,
 compiled for gfx950 on the CPU (about a minute); LOWBIT_ASM_CHECK_ALL=1 checks every GEMM translation unit."""
 import glob
 import os
@@ -50,3 +51,21 @@ def test_the_checker_sees_a_copy_of_a_fresh_accumulator(tmp_path):
     out = subprocess.run([sys.executable, os.path.join(CSRC, "check_gemm_asm.py"), str(bad)], capture_output=True, text=True)
     assert out.returncode == 1
     assert "a41, a16" in out.stdout and "a40, a0" not in out.stdout
+
+
+def test_the_checker_sees_an_mfma_operand_written_right_ahead_of_it(tmp_path):
+    bad = tmp_path / "bad2.s"
+    bad.write_text("_Z16gemm_mfma_kernelv:\n"
+                   "\tv_pk_mul_f16 v3, v20, v21\n"
+                   "\ts_nop 1\n"
+                   "\tv_mfma_f32_32x32x16_f16 a[0:15], v[0:3], v[4:7], a[0:15]\n"      # two wait states: fine
+                   "\tv_pk_mul_f16 v9, v20, v21\n"
+                   "\tds_read_b128 v[30:33], v40\n"
+                   "\tv_mfma_f32_32x32x16_f16 a[16:31], v[8:11], v[4:7], a[16:31]\n"   # one instruction between: not fine
+                   "\tv_pk_mul_f16 v50, v20, v21\n"
+                   "\tv_mfma_f32_32x32x16_f16 a[32:47], v[8:11], v[4:7], a[32:47]\n"   # writes another register: fine
+                   "\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n"
+                   "\ts_endpgm\n")
+    out = subprocess.run([sys.executable, os.path.join(CSRC, "check_gemm_asm.py"), str(bad)], capture_output=True, text=True)
+    assert out.returncode == 1
+    assert out.stdout.count("MFMA operand written by VALU") == 1 and "v9, v20, v21" in out.stdout
