@@ -206,9 +206,10 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     uint32_t xoff[DMA ? 1 : 8];
     int xl[DMA ? 1 : 8];
     // DMA form: x goes global -> LDS without passing through registers, one instruction per piece.  Wave
-    // w fills pieces 8w .. 8w+7: half row w/2, rows 64*(w%2) + 8j ...  Rows past M are clamped (the
-    // offsets are formed with 24-bit multiplies: the launcher keeps M and 2K below 2^24).
-    uint32_t xrow0[2] = {0, 0}, xcol[2] = {0, 0};
+    // w fills pieces 8w .. 8w+7: half row w/2, rows 64*(w%2) + 8j ...  Rows past M are clamped.  Each piece has
+    // its lane offset from the tile's first row in a register of its own (below 2^31: the launcher keeps K
+    // below 2^23), fixed for the whole walk along K; what changes from step to step is a scalar base.
+    uint32_t xone_off[(DMA && MB32 == 4) ? 8 : 1];
     if constexpr (!DMA) {
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -217,13 +218,15 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
             xoff[i] = (uint32_t)(((int64_t)row * K + (wave >> 1) * 64) * (int64_t)sizeof(AT) + xc_l[i & 1]);
             xl[i] = (wave * 8 + i) * 1024 + lane * 16;
         }
-    } else {
+    } else if constexpr (MB32 == 4) {
 #pragma unroll
-        for (int q = 0; q < 2; q++) {
-            xrow0[q] = m0 + (GM / 2) * (wave & 1) + xr_l[q];
-            xcol[q] = (wave >> 1) * 128 + xc_l[q];
+        for (int j = 0; j < 8; j++) {
+            int row = (GM / 2) * (wave & 1) + 8 * j + xr_l[j & 1];
+            row = m0 + row < M ? row : M - 1 - m0;
+            xone_off[j] = (uint32_t)row * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)((wave >> 1) * 128 + xc_l[j & 1]);
         }
     }
+    const uint64_t xone_base = (uint64_t)(uintptr_t)x + (uint64_t)m0 * (uint64_t)K * sizeof(AT);
     constexpr int PW = 8 * MB32 / WAVES;                  // pieces of 1 KiB (8 rows of a half row) a wave fetches per K step
     // Split-K: with a workspace the grid has a second dimension, workgroup (t, s) walks the K steps
     // s * k_steps .. and leaves its fp32 partial tile in ws[s]; a second kernel sums the splits.  It
@@ -239,28 +242,34 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
         // Issued from inline assembly: the compiler's wait-count pass treats an LDS-DMA as aliasing
         // every later LDS access and would wait for it immediately.  Completion is awaited by the
         // explicit vmcnt(0) ahead of the workgroup barrier that publishes the buffer.
-        const uint8_t *xk = (const uint8_t *)x + (int64_t)kt * TILE_COLS * sizeof(AT);
+        const uint64_t src = uniform64(xone_base + (uint64_t)kt * (TILE_COLS * sizeof(AT)));
         const uint32_t lbase = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + wave * PW * 1024);
-        uint32_t row = xrow0[j & 1] + 8 * j;
-        row = row < (uint32_t)M ? row : (uint32_t)M - 1;
-        const uint8_t *src = xk + (__umul24(row, (uint32_t)K * (uint32_t)sizeof(AT)) + xcol[j & 1]);
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                     :: "v"(src), "s"(lbase + j * 1024) : "memory", "m0");
+        asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(xone_off[(DMA && MB32 == 4) ? j : 0]), "s"(src), "s"(lbase), "n"(j * 1024) : "memory", "m0", "scc");
     };
-    // Tall form: the per-lane part of the address is a constant 32-bit offset and everything that changes from
-    // load to load is scalar arithmetic.  Dense launches hand it whole 256-row tiles only, so no row is clamped.
+    // Tall form: the per-lane part of the address is a 32-bit offset, one register per piece (the dense tall form
+    // has registers to spare), and the scalar base changes once per K step: a load is three instructions - M0 from
+    // the buffer's base plus an immediate, the wait state that M0 needs, the load.  (With the piece's rows added to
+    // the scalar base instead it was six, and a load's slot between two MFMAs overran the 28 cycles the MFMA ahead
+    // of it covers.)  Dense launches hand this form whole 256-row tiles only, so no row is clamped.
     const uint32_t xlane_off = (uint32_t)xr_l[0] * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)xc_l[0];       // even pieces
     const uint32_t xlane_off_odd = (uint32_t)xr_l[1] * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)xc_l[1];   // odd pieces
     const uint64_t xwave_base = (uint64_t)(uintptr_t)x +
         ((uint64_t)(m0 + (GM / (WAVES / 2)) * (wave % (WAVES / 2))) * (uint64_t)K + (uint64_t)(wave / (WAVES / 2)) * 64u) * sizeof(AT);
-    auto dma_x_scalar = [&](int kt, uint8_t *buf, int j) __attribute__((always_inline)) {
+    uint32_t xpiece_off[(MB32 == 8 && !GROUPED) ? PW : 1];
+    if constexpr (MB32 == 8 && !GROUPED) {
+#pragma unroll
+        for (int j = 0; j < PW; j++)            // (whole tile below 2^31 bytes from its first row: K < 2^23)
+            xpiece_off[j] = ((j & 1) ? xlane_off_odd : xlane_off) + (uint32_t)j * 8u * (uint32_t)K * (uint32_t)sizeof(AT);
+    }
+    auto dma_x_scalar = [&](int kt, uint8_t *buf, const int j) __attribute__((always_inline)) {
         kt = kt0 + (kt < last ? kt : last);
-        const uint64_t src = xwave_base + (uint64_t)kt * (TILE_COLS * sizeof(AT)) + (uint64_t)j * 8u * (uint64_t)K * sizeof(AT);
+        const uint64_t src = xwave_base + (uint64_t)kt * (TILE_COLS * sizeof(AT));
         const uint32_t lbase = __builtin_amdgcn_readfirstlane(
-            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + (wave * PW + j) * 1024);
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"((j & 1) ? xlane_off_odd : xlane_off), "s"(src), "s"(lbase) : "memory", "m0");
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + wave * PW * 1024);
+        asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(xpiece_off[(MB32 == 8 && !GROUPED) ? j : 0]), "s"(src), "s"(lbase), "n"(j * 1024) : "memory", "m0", "scc");
     };
     // Grouped tall form: a tile holds rows_here <= 256 rows of its group and only the first MBC 32-row blocks are
     // computed.  Wave w fills the pieces 2j + w % 2 (rows 8 * (2j + w % 2) ..) of half row w / 2 for j < 2 * MBC:
