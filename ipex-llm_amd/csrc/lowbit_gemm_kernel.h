@@ -285,22 +285,20 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
         return (uint32_t)row * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)xc_l[wave & 1];
     };
     const uint32_t xlane_off_wave = (wave & 1) ? xlane_off_odd : xlane_off;     // this wave's pieces are all odd or all even
-    auto dma_x_grouped = [&](int kt, uint8_t *buf, int j, auto mbc_, const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
-        constexpr int MBC = decltype(mbc_)::value;
-        kt = kt0 + (kt < last ? kt : last);
-        const bool tail = j >= 2 * (MBC - 1);
-        uint64_t src = xtile_base + (uint64_t)kt * (TILE_COLS * sizeof(AT));
-        if (!tail) src += (uint64_t)(8 * (2 * j + (wave & 1))) * (uint64_t)K * sizeof(AT);
-        // the same in every lane, which the compiler does not always see after the walk over the groups
-        src = uniform64(src);
-        const uint32_t lbase = __builtin_amdgcn_readfirstlane(
-            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + ((wave >> 1) * (4 * MB32) + 2 * j + (wave & 1)) * 1024);
-        const uint32_t voff = tail ? voff_tail[j - 2 * (MBC - 1) < 0 ? 0 : j - 2 * (MBC - 1)] : xlane_off_wave;
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"(voff), "s"(src), "s"(lbase) : "memory", "m0");
-    };
+    // (voff_tail: this lane's offset from the tile's first row for each of the wave's pieces, the rows of the last
+    // block's two clamped; fixed for the walk along K, like the dense forms' - see grouped_piece_offsets below)
     constexpr bool GTALL = GROUPED && MB32 == 8;
-    auto dma_x = [&](int kt, uint8_t *buf, auto mbc_, const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
+    constexpr int NVOFF = GTALL ? 2 * MB32 : 2;
+    auto dma_x_grouped = [&](int kt, uint8_t *buf, const int j, auto mbc_, const uint32_t (&voff_tail)[NVOFF]) __attribute__((always_inline)) {
+        kt = kt0 + (kt < last ? kt : last);
+        // the same in every lane, which the compiler does not always see after the walk over the groups
+        const uint64_t src = uniform64(xtile_base + (uint64_t)kt * (TILE_COLS * sizeof(AT)));
+        const uint32_t lbase = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + ((wave >> 1) * (4 * MB32) + (wave & 1)) * 1024);
+        asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(voff_tail[GTALL ? j : 0]), "s"(src), "s"(lbase), "n"(2 * j * 1024) : "memory", "m0", "scc");
+    };
+    auto dma_x = [&](int kt, uint8_t *buf, auto mbc_, const uint32_t (&voff_tail)[NVOFF]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < (GTALL ? 2 * decltype(mbc_)::value : PW); j++) {
             if constexpr (GTALL) dma_x_grouped(kt, buf, j, mbc_, voff_tail);
@@ -351,7 +349,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     // two waves per SIMD every cycle a wave stands at a memory instruction is a cycle its MFMA pipe idles.
     // `point` = index of the MFMA group (16-column step * row blocks + row block) the call follows.
     auto fetch_units = [&](int kt, uint8_t *buf, WRegs &t, const int point, const int points, auto mbc_,
-                           const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
+                           const uint32_t (&voff_tail)[NVOFF]) __attribute__((always_inline)) {
         constexpr int UNITS = NB32 + (GTALL ? 2 * decltype(mbc_)::value : PW);
         const int spread = points * 5 / 8 > 0 ? points * 5 / 8 : 1;
 #pragma unroll
@@ -367,7 +365,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     // The same for the deeper pipeline of the grouped tall form (below): the pieces of x of step kt_x first, then the
     // weight registers of step kt_w, so that the weight loads are the youngest loads in flight when the step ends.
     auto fetch_units_deep = [&](int kt_x, uint8_t *buf, int kt_w, WRegs &t, const int point, const int points, auto mbc_,
-                                const uint32_t (&voff_tail)[2]) __attribute__((always_inline)) {
+                                const uint32_t (&voff_tail)[NVOFF]) __attribute__((always_inline)) {
         constexpr int XU = GTALL ? 2 * decltype(mbc_)::value : PW, UNITS = XU + NB32;
         const int spread = points * 5 / 8 > 0 ? points * 5 / 8 : 1;
 #pragma unroll
@@ -649,7 +647,13 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                 xtile_base = (uint64_t)lo | ((uint64_t)hi << 32);
                 asm volatile("" : "+v"(wt[0]), "+v"(wt[1]));
             }
-            const uint32_t voff_tail[2] = {tail_offset(2 * (MBC - 1)), tail_offset(2 * (MBC - 1) + 1)};
+            uint32_t voff_tail[NVOFF] = {};               // grouped_piece_offsets
+            if constexpr (GTALL) {
+#pragma unroll
+                for (int j = 0; j < 2 * MBC; j++)
+                    voff_tail[j] = j >= 2 * (MBC - 1) ? tail_offset(j)
+                                                       : xlane_off_wave + (uint32_t)(8 * (2 * j + (wave & 1))) * (uint32_t)K * (uint32_t)sizeof(AT);
+            }
             if constexpr (GTALL && MBC < 8) {
                 // Tiles of a few row blocks have short K steps: with one step of prefetch a step lasted as long as
                 // a weight load takes to come back from HBM, whatever it computed (removing the MFMAs of a four-block
