@@ -218,8 +218,9 @@ int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout,
 static bool ring_range(int qtype, int64_t M, int64_t N, int64_t K) {
     const bool small = (double)M * (double)N * (double)K < 3.5e10;
     if (qtype == LOWBIT_QT_NF4) return small || ((M + 127) / 128) * ((N + 255) / 256) <= 256;
-    // from M = 512 on only while the GEMM's 128-row tiles would cover at most half the machine
-    return small && (M < 512 || (M <= 1024 && ((M + 127) / 128) * ((N + 255) / 256) <= 128));
+    // the other formats: up to 64 rows (its 32- and 64-row tiles), further only on narrow weights; beyond that the
+    // tiled GEMM with its K split is 10-18 % ahead since its epilogue and partial sums became straight-line code
+    return small && (M <= 64 || (M <= 192 && N <= 2048));
 }
 
 size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
@@ -255,13 +256,12 @@ static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, 
     const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
     const int splits = have_ws ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
     const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits);
-    // The ring kernel needs the workspace for its partial tiles; given that, it measured
-    // faster than or level with the tiled GEMM, split or not, below M = 512 (up to 1024 while the GEMM has at
-    // most 128 tiles: [4096 x 4096] at M = 512, 34 against 38 us split) and about 7e10 FLOP (sym_int4 and
-    // sym_int8, seven shapes from [1024 x 8192] to [28672 x 8192]).  With nf4, whose code-book lookups weigh
-    // on the GEMM's tighter loop, it stays ahead at larger M as well while the GEMM's tiles are no more
-    // than one per CU (Llama-3-70B set at M = 512 / 1024: 755 / 808 against 706 / 761 TFLOP/s).  Its own
-    // estimate decides against the GEMV.
+    // The ring kernel needs the workspace for its partial tiles; given that, it measured faster than or level with
+    // the tiled GEMM, split or not, up to M = 64 and on narrow weights (sym_int4, sym_int8, fp8_e4m3; five shapes
+    // from [1024 x 8192] to [28672 x 8192]: [4096 x 4096] at M = 64, 15.5 against 18.0 us; at M = 128 23.0 against
+    // 20.8).  With nf4, whose code-book lookups weigh on the GEMM's tighter loop, it stays ahead at larger M as well
+    // while the GEMM's tiles are no more than one per CU ([11008 x 4096] at M = 256: 47.5 against 59.4 us).  Its
+    // own estimate decides against the GEMV.
     if (have_ws && ring_range(qtype, M, N, K) &&
         ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes)
         return ring_time_us((int)M, (int)N, (int)K, qtype, true) < t_gemv ? PLAN_RING : PLAN_GEMV;
