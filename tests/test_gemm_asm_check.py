@@ -2,8 +2,9 @@
 blocks are still in flight after them.  ipex-llm_amd/csrc/check_gemm_asm.py looks through the generated assembly
 for what that can break (accumulator blocks copied or read too early, scratch memory, function calls, scalar
 base addresses written by the vector unit right ahead of an LDS-DMA, MFMA operands written by the vector unit
-right ahead of the MFMA).  Here it runs on one translation unit,
-compiled for gfx950 on the CPU (about a minute); LOWBIT_ASM_CHECK_ALL=1 checks every GEMM translation unit."""
+right ahead of the MFMA).  Here it runs on three translation units - one grouped format, the dense GEMM, the ring
+kernel - compiled for gfx950 on the CPU (about two minutes); LOWBIT_ASM_CHECK_ALL=1 checks every GEMM translation
+unit."""
 import glob
 import os
 import subprocess
@@ -22,7 +23,7 @@ def _units():
     if os.environ.get("LOWBIT_ASM_CHECK_ALL") == "1":
         return ([os.path.basename(p) for p in sorted(glob.glob(os.path.join(CSRC, "gemm_grouped_*.hip")))]
                 + ["gemm.hip", "gemm_ring.hip"])
-    return ["gemm_grouped_fp8_e4m3.hip", "gemm_ring.hip"]
+    return ["gemm_grouped_fp8_e4m3.hip", "gemm.hip", "gemm_ring.hip"]
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
