@@ -478,6 +478,87 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
         // wave is on its way to a barrier here, the wait is hidden behind it).
         asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 1" : "+a"(acc[MBC - 1][NB32 - 1]));
     };
+    // The same K step for the loop that runs one step ahead (x by LDS-DMA into the other buffer, the other weight
+    // register set), with no seam between steps: a step begins with its first operands in registers.  Behind row
+    // block BMB of its last 16-column step - when every read of this step's buffer has long returned - the step
+    // waits for the next step's loads and passes the workgroup's one barrier per step; what is left of the last
+    // 16-column step then reads the next step's first x operands from the other buffer and dequantizes its first
+    // weights, work that a step otherwise does ahead of its first MFMA with the pipe idle (together with the wait
+    // and the barrier about a tenth of a step).  The last step of a walk does the same (it reads a stale buffer and
+    // dequantizes stale registers into operands nobody uses): one shape of step for the whole loop keeps every
+    // accumulator block in its registers from the first step to the epilogue.
+    auto first_operands = [&](const uint8_t *cur, const WRegs &t, auto mbc_, auto &xv, u32x4 (&wv)[NB32]) __attribute__((always_inline)) {
+        constexpr int MBC = decltype(mbc_)::value;
+#pragma unroll
+        for (int mb = 0; mb < MBC; mb++) xv[mb] = *(const V8 *)(cur + xlane[0] + x_piece(0, mb));
+#pragma unroll
+        for (int nb = 0; nb < NB32; nb++)
+#pragma unroll
+            for (int p = 0; p < 4; p++) wv[nb][p] = dequant_pair(t, 0, nb, p);
+        asm volatile("s_nop 1" : "+v"(wv[0]));          // VALU write of an MFMA operand: two wait states
+        if constexpr (NB32 == 2) asm volatile("" : "+v"(wv[1]));
+    };
+    auto step_ahead = [&](auto &acc, const uint8_t *cur, const uint8_t *nxt, const WRegs &t, const WRegs &tn, auto mbc_,
+                          auto &xv, u32x4 (&wv)[NB32], auto &&between) __attribute__((always_inline)) {
+        constexpr int MBC = decltype(mbc_)::value;
+        constexpr bool HAS_NEXT = true;
+        constexpr int SLOTS = MBC * NB32, PAIRS = 4 * NB32;
+        constexpr bool WAIT_STATES = SLOTS < 4;          // (see compute)
+        constexpr int BMB = MBC > 2 ? 1 : 0;
+        constexpr int TAIL = (MBC - 1 - BMB) * NB32;     // MFMA slots of the last 16-column step behind the barrier
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            u32x4 wn[NB32];
+#pragma unroll
+            for (int mb = 0; mb < MBC; mb++) {
+#pragma unroll
+                for (int nb = 0; nb < NB32; nb++) {
+                    mfma_acc<WAIT_STATES>(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    if (ks < 7) {
+                        const int slot_i = mb * NB32 + nb;
+#pragma unroll
+                        for (int idx = 0; idx < PAIRS; idx++) {
+                            if (idx < (slot_i * PAIRS + SLOTS - 1) / SLOTS || idx >= ((slot_i + 1) * PAIRS + SLOTS - 1) / SLOTS) continue;
+                            wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);
+                        }
+                    } else if constexpr (HAS_NEXT && TAIL > 0) {
+                        if (mb > BMB) {                  // the next step's first weights, over the slots behind the barrier
+                            const int ts = (mb - BMB - 1) * NB32 + nb;
+#pragma unroll
+                            for (int idx = 0; idx < PAIRS; idx++) {
+                                if (idx < (ts * PAIRS + TAIL - 1) / TAIL || idx >= ((ts + 1) * PAIRS + TAIL - 1) / TAIL) continue;
+                                wn[idx >> 2][idx & 3] = dequant_pair(tn, 0, idx >> 2, idx & 3);
+                            }
+                        }
+                    }
+                    if (nb + 1 < NB32 && QT != QT_NF4) __builtin_amdgcn_sched_barrier(0);
+                }
+                if (ks < 7) xv[mb] = *(const V8 *)(cur + xlane[(ks + 1) % 4] + x_piece(ks + 1, mb));
+                else if (HAS_NEXT && mb > BMB) xv[mb] = *(const V8 *)(nxt + xlane[0] + x_piece(0, mb));
+                __builtin_amdgcn_sched_barrier(0);
+                between(ks * MBC + mb, 8 * MBC);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (HAS_NEXT) {
+                    if (ks == 7 && mb == BMB) {
+                        wait_all_loads();                // this wave's part of the next step's x and weights has landed
+                        __syncthreads();                 // (waits for this wave's LDS reads too) the other buffer is complete,
+                                                         // and nobody reads this one any more
+#pragma unroll
+                        for (int m2 = 0; m2 <= BMB; m2++) xv[m2] = *(const V8 *)(nxt + xlane[0] + x_piece(0, m2));
+                        if constexpr (TAIL == 0) {
+#pragma unroll
+                            for (int idx = 0; idx < PAIRS; idx++) wn[idx >> 2][idx & 3] = dequant_pair(tn, 0, idx >> 2, idx & 3);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            if (ks < 7 || HAS_NEXT) {
+#pragma unroll
+                for (int nb = 0; nb < NB32; nb++) wv[nb] = wn[nb];
+            }
+        }
+    };
     typedef std::integral_constant<int, MB32> full_t;
     auto nothing = [](int, int) __attribute__((always_inline)) {};
 
@@ -693,19 +774,22 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
             load_w(0, w0);
             wait_all_loads();
             __syncthreads();
+            w1 = w0;                                     // (never used before it is loaded: a defined value for the last step's look ahead)
+            V8 xv[MBC];
+            u32x4 wv[NB32];
+            first_operands(xs0, w0, mbc, xv, wv);
             for (int kt = 0; kt + 1 < Gs; kt += 2) {
-                compute(acc, xs0, w0, mbc, [&](const int point, const int points) __attribute__((always_inline)) {
+                step_ahead(acc, xs0, xs1, w0, w1, mbc, xv, wv, [&](const int point, const int points) __attribute__((always_inline)) {
                     fetch_units(kt + 1, xs1, w1, point, points, mbc, voff_tail);
                 });
-                wait_all_loads();
-                __syncthreads();
-                compute(acc, xs1, w1, mbc, [&](const int point, const int points) __attribute__((always_inline)) {   // past the end: clamped, unused re-reads
+                step_ahead(acc, xs1, xs0, w1, w0, mbc, xv, wv, [&](const int point, const int points) __attribute__((always_inline)) {   // past the end: clamped, unused re-reads
                     fetch_units(kt + 2, xs0, w0, point, points, mbc, voff_tail);
                 });
-                wait_all_loads();
-                __syncthreads();
             }
-            if (Gs & 1) compute(acc, xs0, w0, mbc, nothing);
+            if (Gs & 1) step_ahead(acc, xs0, xs1, w0, w1, mbc, xv, wv, nothing);
+            // (the compiler may move an accumulator block to other registers where the variants of the loop meet
+            // and does not know that the block written last is still in the MFMA pipe: leave it the time to land)
+            asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 1" : "+a"(acc[MBC - 1][NB32 - 1]));
             epilogue(acc, mbc);
         };
         // tail tiles and small expert groups: 32-row blocks without rows of x skip their MFMAs
