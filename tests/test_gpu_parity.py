@@ -412,3 +412,22 @@ def test_gemm_output_off_16_byte_alignment_equals_aligned_output():
             assert torch.isnan(flat[:shift]).all() and torch.isnan(flat[shift + m * n:]).all()
         with pytest.raises(RuntimeError, match="8-byte aligned"):
             ggml.lowbit_gemm(x.data_ptr(), blob.data_ptr(), y0.data_ptr() + 2, qtype, TILED, DT[dtype], m, n, k, stream())
+
+
+@pytest.mark.gpu
+def test_forward_takes_any_y_alignment_through_the_gemv():
+    """lowbit_forward accepts a y at any 2-byte boundary: the MFMA kernels store 8 bytes and more, so such a y goes
+    through the streaming GEMV in 16-row passes, whatever M."""
+    qtype, dtype, m, n, k = Q4_0, torch.float16, 40, 256, 512
+    w = weights(6600, (n, k))
+    x = acts(6601, m, k, dtype).cuda()
+    blob = dev_quantize(w, qtype, TILED)
+    want = torch.empty((m, n), dtype=dtype, device="cuda")
+    ggml.lowbit_gemv(x.data_ptr(), blob.data_ptr(), want.data_ptr(), qtype, TILED, DT[dtype], m, n, k, 0, stream())
+    flat = torch.full((m * n + 8,), float("nan"), dtype=dtype, device="cuda")
+    y = flat[1:1 + m * n].view(m, n)
+    assert y.data_ptr() % 8 == 2
+    ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), qtype, TILED, DT[dtype], m, n, k, stream())
+    torch.cuda.synchronize()
+    assert torch.equal(y, want)
+    assert torch.isnan(flat[:1]).all() and torch.isnan(flat[1 + m * n:]).all()
