@@ -98,10 +98,15 @@ __device__ inline uint64_t uniform64(uint64_t v) {
     return (uint64_t)lo | ((uint64_t)hi << 32);
 }
 
-// activation of the gate branch: 0 = SiLU, 1 = GELU in its tanh form
+// activation of the gate branch: 0 = SiLU, 1 = GELU in its tanh form.  Written with the hardware's exp2 and
+// reciprocal (1 ulp each; the result is rounded to 16 bits): the correctly rounded division and the library tanh
+// that the build's flags would otherwise expand to are some thirty instructions per value, 128 values per lane in
+// a full tile's epilogue.
 __device__ inline float gemm_gate_act(float g, int act) {
-    if (act == 0) return g / (1.0f + __expf(-g));
-    const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
+    if (act == 0) return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+    const float u = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    // tanh(u) = 1 - 2 / (1 + e^(2u)); e^(2u) = inf gives 1, 0 gives -1
+    const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * u));
     return 0.5f * g * (1.0f + t);
 }
 
