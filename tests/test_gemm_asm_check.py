@@ -2,9 +2,9 @@
 blocks are still in flight after them.  ipex-llm_amd/csrc/check_gemm_asm.py looks through the generated assembly
 for what that can break (accumulator blocks copied or read too early, scratch memory, function calls, scalar
 base addresses written by the vector unit right ahead of an LDS-DMA, MFMA operands written by the vector unit
-right ahead of the MFMA).  Here it runs on three translation units - one grouped format, the dense GEMM, the ring
-kernel - compiled for gfx950 on the CPU (about two minutes); LOWBIT_ASM_CHECK_ALL=1 checks every GEMM translation
-unit."""
+right ahead of the MFMA).  Here it runs on every GEMM translation unit - the grouped formats, the dense GEMM, the
+ring kernel - compiled for gfx950 on the CPU, all at once (two to three minutes on eight cores): the register
+allocation of one format's variant says nothing about another's."""
 import glob
 import os
 import subprocess
@@ -19,19 +19,27 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-packed-fp32-ops", "-S", "--cuda-device-only"]
 
 
-def _units():
-    if os.environ.get("LOWBIT_ASM_CHECK_ALL") == "1":
-        return ([os.path.basename(p) for p in sorted(glob.glob(os.path.join(CSRC, "gemm_grouped_*.hip")))]
-                + ["gemm.hip", "gemm_ring.hip"])
-    return ["gemm_grouped_fp8_e4m3.hip", "gemm.hip", "gemm_ring.hip"]
+UNITS = ([os.path.basename(p) for p in sorted(glob.glob(os.path.join(CSRC, "gemm_grouped_*.hip")))]
+         + ["gemm.hip", "gemm_ring.hip"])
+
+
+@pytest.fixture(scope="module")
+def listings(tmp_path_factory):
+    """unit -> path of its assembly listing (or the compiler's return code), all units compiled concurrently"""
+    out_dir = tmp_path_factory.mktemp("asm")
+    procs = {}
+    for unit in UNITS:
+        listing = str(out_dir / (unit + ".s"))
+        procs[unit] = (listing, subprocess.Popen([HIPCC] + FLAGS + ["-c", os.path.join(CSRC, unit), "-o", listing],
+                                                 cwd=CSRC, stderr=subprocess.DEVNULL))
+    return {unit: (listing if p.wait() == 0 else p.returncode) for unit, (listing, p) in procs.items()}
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
-@pytest.mark.parametrize("unit", _units())
-def test_generated_assembly_respects_the_mfma_hazards(unit, tmp_path):
-    listing = str(tmp_path / (unit + ".s"))
-    subprocess.check_call([HIPCC] + FLAGS + ["-c", os.path.join(CSRC, unit), "-o", listing], cwd=CSRC,
-                          stderr=subprocess.DEVNULL)
+@pytest.mark.parametrize("unit", UNITS)
+def test_generated_assembly_respects_the_mfma_hazards(unit, listings):
+    listing = listings[unit]
+    assert isinstance(listing, str), "hipcc failed on %s with code %s" % (unit, listing)
     # the 128-row DMA form is held to 128 vector registers, for two workgroups per compute unit, and spills a few
     out = subprocess.run([sys.executable, os.path.join(CSRC, "check_gemm_asm.py"), listing, "--allow-scratch", "Lb1ELi4E"],
                          capture_output=True, text=True)
