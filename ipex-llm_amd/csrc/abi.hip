@@ -28,8 +28,8 @@ int launch_gemm_ring(const void *x, const void *w, void *y, int qtype, int act_d
                      void *workspace, size_t workspace_bytes, int wgs, hipStream_t st);
 int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int M, int N, int K,
                 void *workspace, size_t workspace_bytes, int want_splits, hipStream_t st);
-int gemm_splits(int M, int N, int K, size_t ws_bytes);
-double gemm_time_us(int M, int N, int K, int splits);
+int gemm_splits(int M, int N, int K, size_t ws_bytes, int qtype);
+double gemm_time_us(int M, int N, int K, int splits, int qtype);
 int launch_gemv_bf16_f32out(const void *x, const void *w, void *y, int qtype, int layout, int M, int N, int K,
                             hipStream_t st);
 int launch_grouped_gemm(const void *x, const void *const *w, const void *const *w_up, void *y, const int32_t *offsets,
@@ -218,18 +218,23 @@ int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout,
 static bool ring_range(int qtype, int64_t M, int64_t N, int64_t K) {
     const bool small = (double)M * (double)N * (double)K < 3.5e10;
     if (qtype == LOWBIT_QT_NF4) return small || ((M + 127) / 128) * ((N + 255) / 256) <= 256;
-    // the other formats: up to 64 rows (its 32- and 64-row tiles), further only on narrow weights; beyond that the
-    // tiled GEMM with its K split is 10-18 % ahead since its epilogue and partial sums became straight-line code
-    return small && (M <= 64 || (M <= 192 && N <= 2048));
+    // the other formats: up to 64 rows (its 32- and 64-row tiles); beyond that the tiled GEMM with its K split is
+    // level ([1024 x 8192] at M = 96: 19.2 against 18.6 us) or up to 20 % ahead ([2048 x 4096] at M = 192: 18.5
+    // against 22.8 us, [11008 x 4096] at M = 128: 24.8 against 30.2 us)
+    return small && M <= 64;
 }
 
 size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 16 || N <= 0 || K < 128 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;   // M <= 16: GEMV
     if (N % 16 || K % 128) return 0;                                                                  // not tileable: GEMV
     // enough for whichever kernel lowbit_forward_ws may pick for the shape
-    const int s = gemm_splits((int)M, (int)N, (int)K, (size_t)-1);
+    // the query carries no qtype: the most splits and the widest range any format uses
+    int s = 1;
+    for (const int qt : {LOWBIT_QT_SYM_INT4, LOWBIT_QT_SYM_INT8, LOWBIT_QT_NF4}) {
+        const int sq = gemm_splits((int)M, (int)N, (int)K, (size_t)-1, qt);
+        s = sq > s ? sq : s;
+    }
     const size_t gemm = s > 1 ? split_bytes(M, N, s) : 0;
-    // the query carries no qtype: the widest range any format uses
     const size_t ring = ring_range(LOWBIT_QT_NF4, M, N, K) ? ring_workspace_bytes((int)M, (int)N, (int)K, 0) : 0;
     return gemm > ring ? gemm : ring;
 }
@@ -254,12 +259,11 @@ static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, 
     // a pass cannot be shorter than its workgroups' walk along K (narrow weights leave CUs idle)
     const double stream_us = (double)lowbit_blob_bytes(qtype, N * K) / 2.8e6, walk_us = 0.07 * (double)(K / 128);
     const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
-    const int splits = have_ws ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes) : 1;
-    const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits);
+    const int splits = have_ws ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes, qtype) : 1;
+    const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits, qtype);
     // The ring kernel needs the workspace for its partial tiles; given that, it measured faster than or level with
-    // the tiled GEMM, split or not, up to M = 64 and on narrow weights (sym_int4, sym_int8, fp8_e4m3; five shapes
-    // from [1024 x 8192] to [28672 x 8192]: [4096 x 4096] at M = 64, 15.5 against 18.0 us; at M = 128 23.0 against
-    // 20.8).  With nf4, whose code-book lookups weigh on the GEMM's tighter loop, it stays ahead at larger M as well
+    // the tiled GEMM, split or not, up to M = 64 (sym_int4, sym_int8, fp8_e4m3; five shapes from [1024 x 8192] to
+    // [28672 x 8192]: [4096 x 4096] at M = 64, 15.5 against 18.0 us; at M = 128 23.0 against 20.8).  With nf4, whose code-book lookups weigh on the GEMM's tighter loop, it stays ahead at larger M as well
     // while the GEMM's tiles are no more than one per CU ([11008 x 4096] at M = 256: 47.5 against 59.4 us).  Its
     // own estimate decides against the GEMV.
     if (have_ws && ring_range(qtype, M, N, K) &&

@@ -48,40 +48,56 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
     *(at4 *)(y + (int64_t)m * N + n) = o;
 }
 
-// Estimated run time in microseconds of the GEMM with K split `splits` ways (1 = no split), from
-// measurements on MI355X: a workgroup takes about 1.9 us per 128-column step on an otherwise idle
-// machine, 2.7 us when every CU holds one workgroup and 5.0 us when every CU holds two (the clock
-// drops and the memory system fills as more CUs work); the partial sums of a split are written and
-// read back at about 4 TB/s.
-double gemm_time_us(int M, int N, int K, int splits) {
-    const double tiles = (double)((M + GM - 1) / GM) * (double)((N + GN - 1) / GN);
+// A launch of the 128-row DMA form whose tiles leave most compute units idle goes out in half tiles of 64 rows, twice
+// as many workgroups (see the kernel).  Half a tile pays the whole tile's dequantization and takes three quarters of
+// its time per K step.  Measured on sym_int4 fp16 without a workspace, each launch on weights it has not just read:
+// [4096 x 4096] at M = 128 / 512 / 768 (16 / 64 / 96 tiles): 38.9 -> 31.6 / 41.3 -> 34.1 / 41.7 -> 37.4 us;
+// [11008 x 4096] at M = 128 / 256 (43 / 86 tiles): 40.3 -> 33.9 / 41.3 -> 35.8 us; [4096 x 11008] at M = 512:
+// 99.4 -> 82.7 us.  At 112-128 tiles the two are level, and as soon as two halves share a unit it loses: 129 tiles
+// 47 -> 57 us, 256 tiles ([4096 x 4096] at M = 2048) 64 -> 75 us.  Cutting only the tiles of a large launch's last,
+// partly filled round changes nothing (688 tiles: 161 us either way) or loses 2-6 %.
+static bool half_tiles(int M, int64_t tiles, int n_cus) { return M > GM / 2 && tiles * 8 <= (int64_t)n_cus * 3; }
+
+// Estimated run time in microseconds of the GEMM with K split `splits` ways (1 = no split), fitted to measurements on
+// MI355X (sym_int4 fp16, eight weight shapes from [1024 x 8192] to [28672 x 8192], M = 96 .. 1024, 1 .. 8 splits,
+// each launch on weights it has not just read; the fit is within 8 % rms, and the split it picks within 3 % of the
+// best measured one on average, 13 % at worst): a workgroup takes 1.0 us per 128-column step on an otherwise idle
+// machine and 3.3 us when every CU holds two (the clock drops and the memory system fills as more CUs work); launch,
+// prologue and epilogue come to 9.5 us; a workgroup's fp32 partial tile costs 0.035 us to write and sum.  The formats
+// with more work per weight take longer per step (32 tiles of [8192 x 8192] at M = 256 without a split: sym_int4 80,
+// sym_int8 106, nf4 - in the register-staged form that it uses up to one workgroup per CU - 184 us).
+double gemm_time_us(int M, int N, int K, int splits, int qtype) {
+    const int tiles_m = (M + GM - 1) / GM;
+    const double tiles = (double)tiles_m * (double)((N + GN - 1) / GN);
     const int G = K / TILE_COLS;
     const int k_steps = (G + splits - 1) / splits;
     const int ny = (G + k_steps - 1) / k_steps;
-    const double wgs = tiles * ny;
+    const bool halves = ny == 1 && qtype != QT_NF4 && half_tiles(M, (int64_t)tiles, 256);   // (nf4: register-staged form)
+    const double wgs = tiles * ny * (halves ? 2.0 : 1.0);
     const double live = wgs < 512.0 ? wgs : 512.0;
-    // row tiles that are partly empty skip MFMAs and write fewer partial sums: the load-dependent
-    // part of a step and the reduction traffic shrink with the fill, the latency floor does not
-    const double fill = (double)M / ((double)((M + GM - 1) / GM) * GM);
-    const double load = live <= 256.0 ? 0.8 * live / 256.0 : 0.8 + 2.3 * (live - 256.0) / 256.0;
-    const double step = 1.9 + load * (0.4 + 0.6 * fill);
-    double t = (double)k_steps * step * (wgs > 512.0 ? wgs / 512.0 : 1.0);
-    if (ny > 1) t += (double)ny * tiles * (GM * GN * 8.0) * fill / 4.0e6 + 3.0;
+    const double format = qtype == QT_NF4 ? (wgs <= 256.0 ? 2.3 : 1.2) : qtype == QT_SYM_INT8 ? 1.3 : 1.0;
+    const double step = (1.02 + 2.32 * (live / 512.0) * (live / 512.0)) * (halves ? 0.74 : 1.0) * format;
+    // workgroups beyond two per CU wait for a slot: the launch lasts as long as the CU that gets most of them
+    const double rounds = wgs > 512.0 ? (double)(((int64_t)wgs + 255) / 256) / 2.0 : 1.0;
+    double t = 9.5 + (double)k_steps * step * rounds;
+    // row tiles that are partly empty write fewer partial sums
+    const double fill = (double)M / ((double)tiles_m * GM);
+    if (ny > 1) t += 0.035 * (double)ny * tiles * fill;
     return t;
 }
 
 // Number of K splits to use for this shape given `ws_bytes` of workspace (1 = none): the fastest by
 // the estimate above among 1 .. 8 splits of at least two K steps that fit the workspace.
-int gemm_splits(int M, int N, int K, size_t ws_bytes) {
+int gemm_splits(int M, int N, int K, size_t ws_bytes, int qtype) {
     const size_t tiles = (size_t)((M + GM - 1) / GM) * (size_t)((N + GN - 1) / GN);
     const size_t per_split = tiles * GM * GN * sizeof(float);     // whole tiles: partial sums keep the tile layout
     const int G = K / TILE_COLS;
     int best = 1;
-    double best_t = gemm_time_us(M, N, K, 1);
+    double best_t = gemm_time_us(M, N, K, 1, qtype);
     for (int s = 2; s <= 8 && s * 2 <= G; s++) {
         if ((size_t)s * per_split > ws_bytes) break;
-        const double t = gemm_time_us(M, N, K, s);
-        if (t < 0.9 * best_t) {                                   // a split must pay clearly
+        const double t = gemm_time_us(M, N, K, s, qtype);
+        if (t < 0.95 * best_t) {                                  // a split must pay clearly
             best = s;
             best_t = t;
         }
@@ -108,6 +124,11 @@ static int tall_columns(int M, int N, int K, int n_cus, bool heavy_dequant) {
     // it wins with any remainder ([11008 x 4096] at M = 2048: +11 % and +5 %; sym_int4 +1 %, fp8_e4m3 -3 %)
     if (heavy_dequant) return cols;
     return 2 * left >= 3 * n_cus ? cols : 0;
+}
+
+// How many tiles at the end of each XCD's share of a 128-row launch go out as two half tiles: all of them or none.
+static int split_tail_tiles(int M, int64_t tiles, int n_cus) {
+    return half_tiles(M, tiles, n_cus) ? (int)(tiles / 8) + 1 : 0;
 }
 
 // Row tiles per band of the kernel's tile order (see the kernel): the row tiles are cut into at most 8 bands, a
@@ -153,16 +174,18 @@ static int launch_gemm_t(const void *x, const void *w, void *y, int M, int N, in
     const int band_m = band_rows(tiles_m);
     const int k_steps = ws ? (G + splits - 1) / splits : G;
     const int ny = ws ? (G + k_steps - 1) / k_steps : 1;             // splits that actually hold steps
-    dim3 grid(8 * (unsigned)(((int64_t)tiles_m * tiles_n + 7) / 8), ny);
+    const bool fits24 = M < (1 << 24) && K < (1 << 23);              // 24-bit row offsets
+    const bool dma = fits24 && (QT != QT_NF4 || tiles_m * tiles_n * ny > 256);
+    GroupArgs ga{};
+    ga.split_tail = (dma && !ws) ? split_tail_tiles(M, (int64_t)tiles_m * tiles_n, n_cus) : 0;
+    dim3 grid(8 * (unsigned)(((int64_t)tiles_m * tiles_n + 7) / 8 + ga.split_tail), ny);
     // Two forms of the kernel.  The DMA form (x straight into LDS, one K step of prefetch, 128 vector registers)
     // lets a CU hold two workgroups that cover each other's waits, and is 4-8 % ahead with a single workgroup per
     // CU as well - except with nf4, whose code book reads compete with the DMA for LDS: there the register-staged
     // form with its deeper prefetch is 4 % faster while there is at most one workgroup per CU.
-    const bool fits24 = M < (1 << 24) && K < (1 << 23);              // 24-bit row offsets
-    const bool dma = fits24 && (QT != QT_NF4 || tiles_m * tiles_n * ny > 256);
     if (dma)
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
-                           (AT *)y, M, N, K, band_m, GroupArgs{}, k_steps, ws, tn0, tiles_n);
+                           (AT *)y, M, N, K, band_m, ga, k_steps, ws, tn0, tiles_n);
     else
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, false, MB32>), grid, dim3(256), 0, st, (const AT *)x, (const uint8_t *)w,
                            (AT *)y, M, N, K, band_m, GroupArgs{}, k_steps, ws, tn0, tiles_n);
@@ -191,7 +214,7 @@ int launch_gemm(const void *x, const void *w, void *y, int qtype, int layout, in
     if (layout != LAYOUT_TILED || (N % TILE_ROWS) || (K % TILE_COLS) || (((uintptr_t)y) & 7))
         return launch_gemv(x, w, y, qtype, layout, act_dtype, M, N, K, 0, st);
     float *ws = (float *)workspace;
-    const int splits = !ws ? 1 : want_splits > 0 ? want_splits : gemm_splits(M, N, K, workspace_bytes);
+    const int splits = !ws ? 1 : want_splits > 0 ? want_splits : gemm_splits(M, N, K, workspace_bytes, qtype);
     switch (qtype) {
     case QT_SYM_INT4: return launch_gemm_q<QT_SYM_INT4>(x, w, y, act_dtype, M, N, K, ws, splits, st);
     case QT_ASYM_INT4: return launch_gemm_q<QT_ASYM_INT4>(x, w, y, act_dtype, M, N, K, ws, splits, st);

@@ -44,6 +44,8 @@ struct GroupArgs {
     const uint8_t *const *w_up;
     int n_groups;
     int act;                      // activation of the gate branch in the fused form: 0 = SiLU, 1 = tanh-GELU
+    int split_tail;               // dense 128-row DMA form: the last split_tail tiles of every XCD's share go out as two
+                                  // half tiles of 64 rows each, to one workgroup apiece
 };
 
 // Which row tile of which group workgroup `b` of a grouped launch works on.  Whole row tiles come first, then
@@ -154,13 +156,28 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
         const int64_t T = (int64_t)tiles_m * tiles_n;
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
         const int first = (int)(T * xcd / 8), count = (int)(T * (xcd + 1) / 8) - first;
-        if (slot >= count) return;                                                   // whole workgroup leaves
-        const int line = first + slot;
+        // A launch with fewer tiles than compute units goes out in half tiles, twice as many workgroups (the
+        // launcher says how many tiles at the end of each XCD's share are cut: all of them or none).
+        int idx = slot, half = -1;
+        if constexpr (DMA && MB32 == 4) {
+            const int whole = count - (ga.split_tail < count ? ga.split_tail : count);
+            if (slot >= whole) {
+                idx = whole + ((slot - whole) >> 1);
+                half = (slot - whole) & 1;
+            }
+        }
+        if (idx >= count) return;                                                    // whole workgroup leaves
+        const int line = first + idx;
         const int per_band = band_m * tiles_n;
         const int band = line / per_band, r = line - band * per_band;
         const int rows_b = tiles_m - band * band_m < band_m ? tiles_m - band * band_m : band_m;   // the last band may be short
         tile_n = r / rows_b + tn0;
         m0 = (band * band_m + r % rows_b) * GM;
+        if (half >= 0) {
+            m0 += (GM / 2) * half;
+            if (m0 >= M) return;                                                     // (a last row tile of at most 64 rows)
+            M = M < m0 + GM / 2 ? M : m0 + GM / 2;                                   // rows past the half are clamped / not stored
+        }
     } else {
         // every workgroup finds its group by walking the offsets (a handful of scalar loads)
         GroupTile gt;

@@ -390,6 +390,29 @@ def test_gemm_tile_line_covers_every_tile_for_any_tile_counts():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("qtype,dtype", [(Q4_0, torch.float16), (Q4_1, torch.bfloat16), (Q8_0, torch.float16),
+                                         (FP8, torch.bfloat16)])
+def test_gemm_half_tiles_cover_every_row(qtype, dtype):
+    """A launch without a workspace whose tiles leave most compute units idle (at most 96 tiles of 128 x 256) goes
+    out in half tiles of 64 rows.  Row counts on both sides of a half (a last row tile of 1, 64, 65 rows), tile counts
+    on both sides of the limit (96 and 98 tiles), on a y that starts as NaN, against the product with the weights the
+    library's own dequantizer returns (bit-exact against the oracle)."""
+    k = 256
+    for case, (m, n) in enumerate([(65, 512), (128, 2048), (129, 784), (192, 12288), (193, 6144), (320, 8192),
+                                   (200, 12544), (1000, 3072)]):
+        w = weights(6300 + case, (n, k))
+        x = acts(6350 + case, m, k, dtype).cuda()
+        blob = dev_quantize(w, qtype, TILED)
+        want = x.float() @ dev_dequantize(blob, qtype, n, k, TILED, torch.float32).t()
+        y = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        ggml.lowbit_gemm(x.data_ptr(), blob.data_ptr(), y.data_ptr(), qtype, TILED, DT[dtype], m, n, k, stream())
+        torch.cuda.synchronize()
+        assert not torch.isnan(y).any(), (m, n)
+        tol = 2e-3 if dtype == torch.float16 else 8e-3
+        assert (y.float() - want).abs().max() <= tol * want.abs().max(), (m, n)
+
+
+@pytest.mark.gpu
 def test_gemm_output_off_16_byte_alignment_equals_aligned_output():
     """With y 16-byte aligned the GEMM lays a wave's rows out in LDS and stores whole cache lines; any other y takes
     the stores straight from the accumulator layout.  Both must give the same bits, tails in M and N included, in
