@@ -243,7 +243,7 @@ size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 // GEMV streams the weights once per 16 rows of x (about 2.8 TB/s plus 2.5 us per pass; later passes come
 // partly out of the Infinity Cache).  The MFMA GEMM amortizes the dequantization over 128 x 256 tiles
 // but is latency-bound while its tiles do not fill the machine: a lone row tile of [11008 x 4096] takes
-// 61 us however few rows it holds, where a GEMV pass takes 12 us.  With a workspace the GEMM can split
+// 40 us however few rows it holds, where a GEMV pass takes 12 us.  With a workspace the GEMM can split
 // K over more workgroups at the price of writing and re-reading fp32 partial sums, and the ring kernel
 // (32 / 64 / 128-row tiles, units dealt out evenly) covers the batch sizes in between.
 enum { PLAN_GEMV = LOWBIT_PLAN_GEMV, PLAN_RING = LOWBIT_PLAN_RING, PLAN_GEMM = LOWBIT_PLAN_GEMM,
