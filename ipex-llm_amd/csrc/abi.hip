@@ -240,8 +240,8 @@ size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 }
 
 // Choice of kernel behind lowbit_forward, by estimated run time (constants measured on MI355X).  The
-// GEMV streams the weights once per 16 rows of x (about 2.8 TB/s plus 2.5 us per pass; later passes come
-// partly out of the Infinity Cache).  The MFMA GEMM amortizes the dequantization over 128 x 256 tiles
+// GEMV streams the weights once per 16 rows of x (2.8 TB/s for the 4-bit integer formats to 5.8 TB/s for sym_int8,
+// plus 2.5 us per pass; later passes come partly out of the Infinity Cache).  The MFMA GEMM amortizes the dequantization over 128 x 256 tiles
 // but is latency-bound while its tiles do not fill the machine: a lone row tile of [11008 x 4096] takes
 // 40 us however few rows it holds, where a GEMV pass takes 12 us.  With a workspace the GEMM can split
 // K over more workgroups at the price of writing and re-reading fp32 partial sums, and the ring kernel
@@ -257,7 +257,11 @@ static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, 
     if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || K < 128) return PLAN_GEMM;     // reports the error
     const double passes = (double)((M + 15) / 16);
     // a pass cannot be shorter than its workgroups' walk along K (narrow weights leave CUs idle)
-    const double stream_us = (double)lowbit_blob_bytes(qtype, N * K) / 2.8e6, walk_us = 0.07 * (double)(K / 128);
+    // bytes per microsecond of a 16-row pass, measured per format ([11008 x 4096] / [28672 x 8192]-sized weights, two to
+    // eight passes back to back): the formats with more bytes per weight have less to compute per byte
+    const double gemv_rate = qtype == LOWBIT_QT_SYM_INT8 ? 5.8e6 : qtype == LOWBIT_QT_FP8_E4M3 ? 4.7e6
+                             : qtype == LOWBIT_QT_NF4 ? 3.3e6 : 2.8e6;
+    const double stream_us = (double)lowbit_blob_bytes(qtype, N * K) / gemv_rate, walk_us = 0.07 * (double)(K / 128);
     const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
     const int splits = have_ws ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes, qtype) : 1;
     const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits, qtype);

@@ -64,8 +64,9 @@ static bool half_tiles(int M, int64_t tiles, int n_cus) { return M > GM / 2 && t
 // best measured one on average, 13 % at worst): a workgroup takes 1.0 us per 128-column step on an otherwise idle
 // machine and 3.3 us when every CU holds two (the clock drops and the memory system fills as more CUs work); launch,
 // prologue and epilogue come to 9.5 us; a workgroup's fp32 partial tile costs 0.035 us to write and sum.  The formats
-// with more work per weight take longer per step (32 tiles of [8192 x 8192] at M = 256 without a split: sym_int4 80,
-// sym_int8 106, nf4 - in the register-staged form that it uses up to one workgroup per CU - 184 us).
+// with more work per weight take longer per step (per step of a launch of a few dozen tiles, without a split:
+// sym_int4 1.03 us, fp8_e4m3 1.30, sym_int8 1.47, nf4 - in the register-staged form that it uses up to one workgroup
+// per CU - 2.7).
 double gemm_time_us(int M, int N, int K, int splits, int qtype) {
     const int tiles_m = (M + GM - 1) / GM;
     const double tiles = (double)tiles_m * (double)((N + GN - 1) / GN);
@@ -75,8 +76,10 @@ double gemm_time_us(int M, int N, int K, int splits, int qtype) {
     const bool halves = ny == 1 && qtype != QT_NF4 && half_tiles(M, (int64_t)tiles, 256);   // (nf4: register-staged form)
     const double wgs = tiles * ny * (halves ? 2.0 : 1.0);
     const double live = wgs < 512.0 ? wgs : 512.0;
-    const double format = qtype == QT_NF4 ? (wgs <= 256.0 ? 2.3 : 1.2) : qtype == QT_SYM_INT8 ? 1.3 : 1.0;
-    const double step = (1.02 + 2.32 * (live / 512.0) * (live / 512.0)) * (halves ? 0.74 : 1.0) * format;
+    const double format = qtype == QT_NF4 ? (wgs <= 256.0 ? 2.4 : 1.2) : qtype == QT_SYM_INT8 ? 1.4 : qtype == QT_FP8_E4M3 ? 1.25 : 1.0;
+    // (half a tile repeats the tile's dequantization: the formats that pay most for it gain 3-13 % instead of 15-25 %)
+    const double half = !halves ? 1.0 : (qtype == QT_SYM_INT8 || qtype == QT_FP8_E4M3) ? 0.92 : 0.74;
+    const double step = (1.02 + 2.32 * (live / 512.0) * (live / 512.0)) * half * format;
     // workgroups beyond two per CU wait for a slot: the launch lasts as long as the CU that gets most of them
     const double rounds = wgs > 512.0 ? (double)(((int64_t)wgs + 255) / 256) / 2.0 : 1.0;
     double t = 9.5 + (double)k_steps * step * rounds;
