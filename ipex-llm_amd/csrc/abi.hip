@@ -261,7 +261,7 @@ static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, 
     // eight passes back to back): the formats with more bytes per weight have less to compute per byte
     const double gemv_rate = qtype == LOWBIT_QT_SYM_INT8 ? 5.8e6 : qtype == LOWBIT_QT_FP8_E4M3 ? 4.7e6
                              : qtype == LOWBIT_QT_NF4 ? 3.3e6 : 2.8e6;
-    const double stream_us = (double)lowbit_blob_bytes(qtype, N * K) / gemv_rate, walk_us = 0.07 * (double)(K / 128);
+    const double stream_us = (double)lowbit_blob_bytes(qtype, N * K) / gemv_rate, walk_us = (qtype == LOWBIT_QT_NF4 ? 0.14 : 0.10) * (double)(K / 128);
     const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
     const int splits = have_ws ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes, qtype) : 1;
     const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits, qtype);

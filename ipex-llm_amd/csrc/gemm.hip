@@ -90,14 +90,16 @@ double gemm_time_us(int M, int N, int K, int splits, int qtype) {
 }
 
 // Number of K splits to use for this shape given `ws_bytes` of workspace (1 = none): the fastest by
-// the estimate above among 1 .. 8 splits of at least two K steps that fit the workspace.
+// the estimate above among 1 .. 16 splits of at least two K steps that fit the workspace (more than 8 pay on long K
+// with few tiles: fp8_e4m3 [4096 x 14336] at M = 128: 12 splits 33.6 us, 8 splits 35.4; sym_int8 [1024 x 8192]: 16
+// splits 20.0, 8 splits 22.7).
 int gemm_splits(int M, int N, int K, size_t ws_bytes, int qtype) {
     const size_t tiles = (size_t)((M + GM - 1) / GM) * (size_t)((N + GN - 1) / GN);
     const size_t per_split = tiles * GM * GN * sizeof(float);     // whole tiles: partial sums keep the tile layout
     const int G = K / TILE_COLS;
     int best = 1;
     double best_t = gemm_time_us(M, N, K, 1, qtype);
-    for (int s = 2; s <= 8 && s * 2 <= G; s++) {
+    for (int s = 2; s <= 16 && s * 2 <= G; s++) {
         if ((size_t)s * per_split > ws_bytes) break;
         const double t = gemm_time_us(M, N, K, s, qtype);
         if (t < 0.95 * best_t) {                                  // a split must pay clearly

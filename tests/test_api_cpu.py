@@ -318,7 +318,7 @@ def test_kernel_choice_boundaries_are_pinned():
         (2, 4096, 11008):  ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, M, M, M, M, M, M]),
         (3, 11008, 4096):  ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
         (10, 8192, 8192):  ([G, G, R, R, R, R, R, R, R, R, M], [G, G, G, G, G, G, M, M, M, M, M]),
-        (10, 1024, 8192):  ([G, G, G, G, R, R, R, R, R, R, R], [G, G, G, G, G, G, G, M, M, M, M]),
+        (10, 1024, 8192):  ([G, G, R, R, R, R, R, R, R, R, R], [G, G, G, G, G, G, M, M, M, M, M]),
         (10, 28672, 8192): ([G, G, R, R, R, R, R, M, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
         (10, 8192, 28672): ([G, G, R, R, R, R, R, R, R, R, M], [G, G, G, G, G, G, M, M, M, M, M]),
         (8, 28672, 8192):  ([G, G, R, R, R, S, M, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),

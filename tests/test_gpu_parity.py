@@ -301,7 +301,7 @@ def test_llama3_70b_shapes_decode_against_oracle(qtype, n, k, m):
 
 @pytest.mark.parametrize("qtype,dtype", [(Q4_0, torch.float16), (Q8_0, torch.bfloat16), (NF4, torch.bfloat16)])
 @pytest.mark.parametrize("m,n,k,splits", [(48, 1024, 4096, 8), (200, 272, 1408, 3), (512, 4096, 2048, 2),
-                                          (130, 11008, 1024, 4), (300, 7168, 896, 7)])
+                                          (130, 11008, 1024, 4), (300, 7168, 896, 7), (96, 512, 4096, 16)])
 def test_split_k_gemm_against_oracle(qtype, dtype, m, n, k, splits):
     # K split over several workgroups per tile, partial sums through a workspace; ragged splits
     # (11 steps in 3, 7 steps in 7), both forms of the kernel, tail row tiles
