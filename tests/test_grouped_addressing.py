@@ -3,7 +3,8 @@ grouped_tile, dma_x_grouped, the LDS piece layout), checked for what must hold w
 every (group, row tile, column tile) is worked on exactly once; every byte the LDS-DMA fetches lies inside x
 (the rows of the last 32-row block are clamped to the group's last row); every 16-byte operand that the MFMAs of
 the computed blocks read from LDS has been filled with the row and columns it stands for; loads take whole cache
-lines per eight lanes and operand reads spread over all LDS banks."""
+lines per eight lanes and operand reads spread over all LDS banks.  At the end: the dense 128-row form's line of tiles,
+dealt to the XCDs whole or in 64-row halves, covers every row of every column tile exactly once."""
 import numpy as np
 import pytest
 
@@ -138,3 +139,62 @@ def test_random_row_counts():
     rng = np.random.default_rng(0)
     for _ in range(25):
         check([int(v) for v in rng.integers(0, 600, size=rng.integers(1, 9))], 4096, tiles_n=2)
+
+
+# ---- dense 128-row form: the line of tiles dealt to the XCDs, whole or in 64-row halves (lowbit_gemm_kernel.h,
+# the !GROUPED branch at the top of gemm_mfma_kernel; gemm.hip: band_rows, split_tail_tiles and the grid)
+
+def _band_rows(tiles_m):
+    bands = 1
+    while bands * 2 <= 8 and bands * 2 <= tiles_m:
+        bands *= 2
+    return (tiles_m + bands - 1) // bands
+
+
+def _dense_rows_covered(M, tiles_n, split_tail):
+    """rows of y that each (row, column tile) receives, from every workgroup of the launch"""
+    GM = 128
+    tiles_m = (M + GM - 1) // GM
+    T = tiles_m * tiles_n
+    band_m = _band_rows(tiles_m)
+    grid = 8 * ((T + 7) // 8 + split_tail)
+    hits = np.zeros((M, tiles_n), dtype=np.int32)
+    for b in range(grid):
+        xcd, slot = b & 7, b >> 3
+        first = T * xcd // 8
+        count = T * (xcd + 1) // 8 - first
+        idx, half = slot, -1
+        whole = count - min(split_tail, count)
+        if slot >= whole:
+            idx = whole + ((slot - whole) >> 1)
+            half = (slot - whole) & 1
+        if idx >= count:
+            continue
+        line = first + idx
+        per_band = band_m * tiles_n
+        band, r = divmod(line, per_band)
+        rows_b = min(tiles_m - band * band_m, band_m)
+        tile_n = r // rows_b
+        m0 = (band * band_m + r % rows_b) * GM
+        m_end = M
+        if half >= 0:
+            m0 += (GM // 2) * half
+            if m0 >= M:
+                continue
+            m_end = min(M, m0 + GM // 2)
+        else:
+            m_end = min(M, m0 + GM)
+        assert 0 <= tile_n < tiles_n and 0 <= m0 < M
+        hits[m0:m_end, tile_n] += 1
+    return hits
+
+
+def test_dense_tile_line_with_half_tiles_covers_every_row_once():
+    rng = np.random.default_rng(5)
+    cases = [(65, 2), (128, 8), (129, 3), (192, 48), (193, 24), (64, 5), (1, 1), (2048, 43), (1000, 12)]
+    cases += [(int(rng.integers(1, 1500)), int(rng.integers(1, 50))) for _ in range(40)]
+    for M, tiles_n in cases:
+        T = (M + 127) // 128 * tiles_n
+        for split_tail in (0, T // 8 + 1, 3):          # none, all (what the launcher passes), a few at each share's end
+            hits = _dense_rows_covered(M, tiles_n, split_tail)
+            assert (hits == 1).all(), (M, tiles_n, split_tail)
