@@ -40,26 +40,55 @@ class MergedProjectionSlice(torch.nn.Module):
     is a valid weight.  The slice owns no parameters; the attention module is kept as a plain attribute, not as
     a registered sub-module, so that the module tree has no cycle through it."""
 
-    def __init__(self, owner: torch.nn.Module, start: int, length: int, leader: bool):
+    def __init__(self, owner: torch.nn.Module, start: int, length: int, leader: bool, last: bool = False):
         super().__init__()
         self.__dict__["_owner"] = owner
-        self.start, self.length, self.leader = start, length, leader
+        self.start, self.length, self.leader, self.last = start, length, leader, last
         self.out_features = length
 
     @property
     def in_features(self):
         return self._owner.qkv_proj.in_features
 
+    @property
+    def weight(self):
+        """This slice's rows of a dense merged weight; the merged low-bit parameter itself otherwise (callers
+        read `.dtype` / `.device` of it, as they would of a `LowBitLinear`'s packed weight)."""
+        w = self._owner.qkv_proj.weight
+        if getattr(w, "quantized", False) or w.dim() != 2 or w.size(0) < self.start + self.length:
+            return w
+        return w[self.start:self.start + self.length]
+
+    @property
+    def bias(self):
+        b = self._owner.qkv_proj.bias
+        return None if b is None else b[self.start:self.start + self.length]
+
     def forward(self, x: torch.Tensor):
         owner = self._owner
-        cache = getattr(owner, "_qkv_cache", None)
-        if cache is not None and cache[0]() is x and cache[1] == x._version:
-            return cache[2][..., self.start:self.start + self.length]
-        if self.leader:
-            y = owner.qkv_proj(x)
-            owner._qkv_cache = (weakref.ref(x), x._version, y)
+        cache = owner.__dict__.get("_qkv_cache")
+        if cache is not None and cache[0]() is x and cache[1] == _version_of(x):
+            y = cache[2]
+            if self.last:
+                owner.__dict__["_qkv_cache"] = None        # q, k and v have read it: nothing is kept alive
             return y[..., self.start:self.start + self.length]
-        return _project_rows(owner.qkv_proj, x, self.start, self.length)
+        if not self.leader:
+            if cache is not None:
+                # the merged product was run on another tensor (cross-attention): from now on the leader
+                # computes its own rows only
+                owner.__dict__["_qkv_cache"] = None
+                owner.__dict__["_qkv_apart"] = True
+            return _project_rows(owner.qkv_proj, x, self.start, self.length)
+        if owner.__dict__.get("_qkv_apart", False):
+            return _project_rows(owner.qkv_proj, x, self.start, self.length)
+        y = owner.qkv_proj(x)
+        owner.__dict__["_qkv_cache"] = (weakref.ref(x), _version_of(x), y)
+        return y[..., self.start:self.start + self.length]
+
+
+def _version_of(x: torch.Tensor) -> int:
+    """In-place edits bump `_version`; inference tensors do not count them (reading it raises)."""
+    return 0 if x.is_inference() else x._version
 
 
 def _project_rows(linear: torch.nn.Module, x: torch.Tensor, start: int, length: int):
@@ -76,6 +105,8 @@ def _project_rows(linear: torch.nn.Module, x: torch.Tensor, start: int, length: 
                         layout=w.blob_layout)
         y = y.view(*x.shape[:-1], length)
         return y if bias is None else y + bias.to(y.dtype)
+    if type(linear) is torch.nn.Linear:
+        return torch.nn.functional.linear(x, linear.weight[start:start + length], bias)
     return linear(x)[..., start:start + length]
 
 
@@ -99,7 +130,7 @@ def merge_qkv_base(module: torch.nn.Module, attention_class):
             module.qkv_proj = qkv_proj
             start = 0
             for i, (name, size) in enumerate(zip(("q_proj", "k_proj", "v_proj"), sizes)):
-                setattr(module, name, MergedProjectionSlice(module, start, size, leader=(i == 0)))
+                setattr(module, name, MergedProjectionSlice(module, start, size, leader=(i == 0), last=(i == 2)))
                 start += size
 
 

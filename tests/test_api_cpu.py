@@ -257,6 +257,45 @@ def test_optimize_pre_merges_qkv_and_the_stock_attention_forward_still_works():
     assert _optimize_pre(gpt) is gpt
 
 
+def test_merged_qkv_slices_under_inference_mode_and_cache_lifetime():
+    """Inference tensors carry no version counter; the merged product is dropped once q, k and v have read
+    it; a model whose k/v see another tensor than q (cross-attention) stops running the merged product;
+    stock attention code reads `q_proj.weight.dtype` and `q_proj.bias`."""
+    transformers = pytest.importorskip("transformers")
+    from ipex_llm.transformers.convert import _optimize_pre
+    cfg = transformers.LlamaConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=50,
+                                   max_position_embeddings=32, attention_bias=True)
+    torch.manual_seed(4)
+    model = transformers.LlamaForCausalLM(cfg).eval()
+    ids = torch.randint(0, 50, (2, 7))
+    with torch.no_grad():
+        want = model(ids).logits
+    attn = model.model.layers[0].self_attn
+    wq, wk, bq = attn.q_proj.weight.detach().clone(), attn.k_proj.weight.detach().clone(), attn.q_proj.bias.detach().clone()
+    model = _optimize_pre(model)
+    with torch.inference_mode():
+        got = model(ids).logits
+        out = model.generate(ids, max_new_tokens=3, do_sample=False)
+    assert torch.allclose(got, want, atol=1e-5, rtol=1e-5) and out.shape == (2, 10)
+    for layer in model.model.layers:
+        assert layer.self_attn.__dict__.get("_qkv_cache") is None          # no activation stays pinned
+    attn = model.model.layers[0].self_attn
+    assert attn.q_proj.weight.dtype == torch.float32 and torch.equal(attn.q_proj.weight, wq)
+    assert torch.equal(attn.k_proj.weight, wk) and torch.equal(attn.q_proj.bias, bq)
+    # cross-attention: q on one tensor, k and v on another
+    calls = []
+    inner = attn.qkv_proj.forward
+    attn.qkv_proj.forward = lambda t: (calls.append(t.shape), inner(t))[1]
+    a, b = torch.randn(3, 64), torch.randn(5, 64)
+    with torch.inference_mode():
+        for _ in range(2):
+            q, k, v = attn.q_proj(a), attn.k_proj(b), attn.v_proj(b)
+    assert torch.allclose(q, a @ wq.t() + bq, atol=1e-5) and torch.allclose(k, b @ wk.t() + attn.k_proj.bias, atol=1e-5)
+    assert v.shape == (5, 32) and attn.__dict__["_qkv_cache"] is None and attn.__dict__["_qkv_apart"]
+    assert len(calls) == 1             # merged once; every later call multiplies its own rows only
+
+
 def test_linears_whose_row_length_is_no_multiple_of_the_block_stay_dense():
     # fp8_e4m3 blocks hold 128 weights: 192 input features pass the reference's % 64 rule but cannot be quantized
     with torch.device("meta"):

@@ -200,6 +200,31 @@ def test_from_pretrained_tiny_llama_and_low_bit_round_trip(tmp_path):
     assert torch.equal(got, got2)
 
 
+def test_tiny_llama_generates_under_inference_mode(tmp_path):
+    """Callers of the reference run `generate` inside `torch.inference_mode()`: activations are inference
+    tensors there (no version counter) and nothing of a layer's merged q/k/v product may outlive the layer."""
+    transformers = pytest.importorskip("transformers")
+    from ipex_llm.transformers import AutoModelForCausalLM
+    cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=320,
+                                   max_position_embeddings=64)
+    torch.manual_seed(6)
+    hf = transformers.LlamaForCausalLM(cfg).eval()
+    src = tmp_path / "fp"
+    hf.save_pretrained(str(src))
+    model = AutoModelForCausalLM.from_pretrained(str(src), load_in_low_bit="sym_int4").to("cuda")
+    ids = torch.randint(0, 320, (2, 9)).cuda()
+    with torch.no_grad():
+        want = model(ids).logits
+        tokens_want = model.generate(ids, max_new_tokens=4, do_sample=False)
+    with torch.inference_mode():
+        got = model(ids).logits
+        tokens = model.generate(ids, max_new_tokens=4, do_sample=False)
+    assert torch.equal(got, want) and torch.equal(tokens, tokens_want) and tokens.shape == (2, 13)
+    for layer in model.model.layers:
+        assert layer.self_attn.__dict__.get("_qkv_cache") is None
+
+
 @pytest.mark.parametrize("qname,dtype", [("nf4", torch.bfloat16), ("sym_int4", torch.float16)])
 def test_training_backward_is_grad_out_times_the_dequantized_weight(qname, dtype):
     """MatMulLowBit.backward (reference: low_bit_linear.py:520-541), the QLoRA gradient path."""
