@@ -281,6 +281,12 @@ size_t lowbit_grouped_workspace_bytes(int n_groups, int64_t total_rows, int64_t 
 int lowbit_grouped_forward_ws(const void *x, const void *const *w, void *y, const int32_t *group_offsets,
                               int n_groups, int64_t total_rows, int qtype, int act_dtype, int64_t N, int64_t K,
                               void *workspace, size_t workspace_bytes, void *stream);
+/* Host arithmetic only (no GPU call, like lowbit_forward_plan): how lowbit_grouped_forward(_ws) would run the
+ * shape.  plan4 = {256-row tiles (1) or 128-row tiles (0), K splits, waves per workgroup, workgroups per split}.
+ * Every workgroup of a split launch owns one 256 x 256 fp32 tile of the workspace: splits x workgroups x 256 KiB
+ * never exceeds lowbit_grouped_workspace_bytes.  No counterpart in the reference (its expert loop has no plan). */
+int lowbit_grouped_forward_plan(int n_groups, int64_t total_rows, int64_t N, int64_t K, int have_workspace,
+                                size_t workspace_bytes, int *plan4);
 /* The gated MLP's first half for all experts in one launch: rows of group e of y [total_rows, N] =
  * act(x w_gate[e]^T) .* (x w_up[e]^T), act as in lowbit_mlp_forward.  It is what the per-expert loop computes
  * with two LowBitLinear calls and an activation per expert

@@ -36,6 +36,7 @@ int launch_grouped_gemm(const void *x, const void *const *w, const void *const *
                         int n_groups, int total_rows, int qtype, int act_dtype, int N, int K, int act, void *workspace,
                         size_t workspace_bytes, hipStream_t st);
 size_t grouped_workspace_bytes(int total_rows, int n_groups, int N, int K);
+void grouped_plan_query(int total_rows, int n_groups, int N, int K, size_t ws_bytes, int out[4]);
 }  // namespace lowbit
 
 using namespace lowbit;
@@ -483,6 +484,15 @@ size_t lowbit_grouped_workspace_bytes(int n_groups, int64_t total_rows, int64_t 
     if (n_groups <= 0 || total_rows <= 0 || total_rows > 0x7fffffff || N <= 0 || K <= 0 || N > 0x7fffffff || K > 0x7fffffff)
         return 0;
     return grouped_workspace_bytes((int)total_rows, n_groups, (int)N, (int)K);
+}
+
+int lowbit_grouped_forward_plan(int n_groups, int64_t total_rows, int64_t N, int64_t K, int have_workspace,
+                                size_t workspace_bytes, int *plan4) {
+    if (!plan4 || n_groups <= 0 || total_rows <= 0 || total_rows > 0x7fffffff || N <= 0 || K < 128 || N > 0x7fffffff ||
+        K > 0x7fffffff)
+        return fail(LOWBIT_EARG, "lowbit_grouped_forward_plan: bad argument");
+    grouped_plan_query((int)total_rows, n_groups, (int)N, (int)K, have_workspace ? workspace_bytes : 0, plan4);
+    return 0;
 }
 
 int lowbit_grouped_forward_ws(const void *x, const void *const *w, void *y, const int32_t *group_offsets, int n_groups,

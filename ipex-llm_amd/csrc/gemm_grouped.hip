@@ -18,16 +18,10 @@
 // gemm_grouped_<format>.hip from lowbit_gemm_grouped.h).
 #include <hip/hip_runtime.h>
 #include "lowbit_formats.h"
+#include "lowbit_grouped_plan.h"
 
 namespace lowbit {
 
-// the tile sizes of lowbit_gemm_kernel.h that the choices below depend on
-constexpr int G_GN = 256, G_GM_TALL = 256;
-
-struct GroupedPlan {
-    bool tall;
-    int splits;
-};
 template <int QT>
 int launch_grouped_q(const void *x, const void *const *w, const void *const *w_up, void *y, const int32_t *offsets,
                      int n_groups, int total_rows, int dt, int N, int K, int act, const GroupedPlan &plan, float *ws,
@@ -43,9 +37,15 @@ static int device_cus() {
     return n_cus;
 }
 
+// Bytes of workspace per K split of the tall form: a partial tile per workgroup of the launch, whichever of the two
+// tile orders it takes (the grid, and with it a workgroup's slot in the workspace, depends on the order).
+static int tall_grid(int total_rows, int n_groups, int tiles_n, bool one_round) {
+    return grouped_grid(grouped_max_row_tiles(total_rows, n_groups, G_GM_TALL), tiles_n, grouped_chunk(tiles_n, one_round));
+}
 static size_t tall_split_bytes(int total_rows, int n_groups, int N) {
     const int tiles_n = (N + G_GN - 1) / G_GN;
-    return (size_t)tiles_n * (total_rows / G_GM_TALL + n_groups) * G_GM_TALL * G_GN * sizeof(float);
+    const int a = tall_grid(total_rows, n_groups, tiles_n, false), b = tall_grid(total_rows, n_groups, tiles_n, true);
+    return (size_t)(a > b ? a : b) * G_GM_TALL * G_GN * sizeof(float);
 }
 
 // Form and K splits for a grouped product given `ws_bytes` of workspace.  Measured on MI355X (8 groups of
@@ -55,6 +55,24 @@ static size_t tall_split_bytes(int total_rows, int n_groups, int N) {
 //     projection) that beats both unsplit forms at every row count (32 rows per group: 131 against 193 us).
 //   - Otherwise the 128-row form with two workgroups per unit is ahead up to about 96 rows per group (147
 //     against 156 us at 96) and the tall form from there on (108-150 rows per group: 195 against 245 us).
+// Waves per workgroup of the tall form.  Eight (32 weight rows each, two per SIMD) cover part of each other's waits
+// where a tile has few MFMAs per weight: measured on MI355X with eight groups of 110-151 rows of fp8_e4m3 weights,
+// the fused gate/up launch ([14336 x 4096] twice) takes 341-352 us with eight waves against 372-375 with four; the
+// plain product of the down projection ([4096 x 14336], two K splits) 169 against 153-156 - its workgroups are a
+// single round, and eight waves read every x operand from LDS twice as often.
+static int grouped_waves(int total_rows, int n_groups, bool fused) {
+    return fused && (int64_t)total_rows <= (int64_t)n_groups * 192 ? 8 : 4;
+}
+
+// Whether the workgroups that hold rows (an estimate: the host never sees the offsets) all run at once: the tall
+// form holds one workgroup per compute unit, the 128-row form two.  The tile order then keeps a row tile's column
+// tiles on one XCD (see grouped_tile) - when there are row tiles for every XCD.
+static bool grouped_one_round(int total_rows, int n_groups, int tiles_n, bool tall, int splits) {
+    const int rows = tall ? G_GM_TALL : G_GM_TALL / 2;
+    const int row_tiles = total_rows / rows > n_groups ? total_rows / rows : n_groups;
+    return row_tiles >= 8 && (int64_t)row_tiles * tiles_n * splits <= (int64_t)device_cus() * (tall ? 1 : 2);
+}
+
 GroupedPlan grouped_plan(int total_rows, int n_groups, int N, int K, size_t ws_bytes) {
     const int tiles_n = (N + G_GN - 1) / G_GN, G = K / TILE_COLS;
     const int row_tiles = total_rows / G_GM_TALL > n_groups ? total_rows / G_GM_TALL : n_groups;   // estimate of the tiles that hold rows
@@ -64,7 +82,19 @@ GroupedPlan grouped_plan(int total_rows, int n_groups, int N, int K, size_t ws_b
     const size_t per_split = tall_split_bytes(total_rows, n_groups, N);
     while (s > 1 && (size_t)s * per_split > ws_bytes) s--;
     if (s < 1) s = 1;
-    return {s > 1 || (int64_t)total_rows > (int64_t)n_groups * 96, s};
+    const bool tall = s > 1 || (int64_t)total_rows > (int64_t)n_groups * 96;
+    return {tall, s, grouped_waves(total_rows, n_groups, false), grouped_one_round(total_rows, n_groups, tiles_n, tall, s)};
+}
+
+// What launch_grouped_gemm would do for a plain grouped product: {tall, splits, waves, grid.x}.
+void grouped_plan_query(int total_rows, int n_groups, int N, int K, size_t ws_bytes, int out[4]) {
+    const GroupedPlan p = grouped_plan(total_rows, n_groups, N, K, ws_bytes);
+    const int tiles_n = (N + G_GN - 1) / G_GN;
+    out[0] = p.tall;
+    out[1] = p.splits;
+    out[2] = p.tall ? p.waves : 4;
+    out[3] = p.tall ? tall_grid(total_rows, n_groups, tiles_n, p.one_round)
+                    : grouped_grid(grouped_max_row_tiles(total_rows, n_groups, G_GM_TALL / 2), tiles_n, grouped_chunk(tiles_n, p.one_round));
 }
 
 size_t grouped_workspace_bytes(int total_rows, int n_groups, int N, int K) {
@@ -80,7 +110,9 @@ int launch_grouped_gemm(const void *x, const void *const *w, const void *const *
     if (total_rows == 0 || N == 0 || n_groups == 0) return 0;
     if (total_rows >= (1 << 24) || K >= (1 << 23)) return -3;        // 24-bit row offsets in the kernel
     float *ws = (float *)workspace;
-    const GroupedPlan plan = w_up ? GroupedPlan{true, 1} : grouped_plan(total_rows, n_groups, N, K, ws ? workspace_bytes : 0);
+    const GroupedPlan plan = w_up ? GroupedPlan{true, 1, grouped_waves(total_rows, n_groups, true),
+                                                grouped_one_round(total_rows, n_groups, (N + G_GN / 2 - 1) / (G_GN / 2), true, 1)}
+                                  : grouped_plan(total_rows, n_groups, N, K, ws ? workspace_bytes : 0);
     switch (qtype) {
     case QT_SYM_INT4: return launch_grouped_q<QT_SYM_INT4>(x, w, w_up, y, offsets, n_groups, total_rows, act_dtype, N, K, act, plan, ws, st);
     case QT_ASYM_INT4: return launch_grouped_q<QT_ASYM_INT4>(x, w, w_up, y, offsets, n_groups, total_rows, act_dtype, N, K, act, plan, ws, st);

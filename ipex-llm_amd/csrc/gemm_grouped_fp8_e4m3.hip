@@ -7,3 +7,4 @@ template int launch_grouped_q<QT_FP8_E4M3>(const void *, const void *const *, co
                                     int, int, int, int, const GroupedPlan &, float *, hipStream_t);
 
 }  // namespace lowbit
+

@@ -173,4 +173,5 @@ template <bool NOP = true> __device__ inline void mfma_acc(f32x16 &c, bf16x8 a, 
     else asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
+
 }  // namespace lowbit

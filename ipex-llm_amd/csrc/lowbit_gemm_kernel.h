@@ -13,6 +13,7 @@
 //   and stores 8 contiguous bytes of y at a time.
 #pragma once
 #include "lowbit_gemm.h"
+#include "lowbit_grouped_plan.h"
 
 namespace lowbit {
 
@@ -34,8 +35,10 @@ constexpr int GM_TALL = 256, MB32_TALL = GM_TALL / 32;
 // tall form dequantizes every weight once per 256 rows of x: half the VALU work, half the weight loads and
 // half the barriers per MFMA; its 16 accumulator blocks take all 256 accumulation registers, so a CU holds
 // one workgroup.  tn0 / tn_cnt: the launch covers the column tiles tn0 .. tn0 + tn_cnt - 1 of y.
-// WAVES = 8 (dense tall form only): the same tile with eight waves of 32 weight rows, two per SIMD, 128
-// accumulation registers each; every x operand read from LDS then feeds one MFMA instead of two.
+// WAVES = 8 (tall form only): the same tile with eight waves of 32 weight rows, two per SIMD, 128
+// accumulation registers each; every x operand read from LDS then feeds one MFMA instead of two.  The two waves
+// of a SIMD cover each other's dequantization, LDS reads and barrier waits, which a partly filled grouped tile
+// (a few 32-row blocks of x: few MFMAs per weight) cannot cover with its own MFMAs.
 // Grouped mode (mixture-of-experts): rows offsets[e] .. offsets[e+1]-1 of x use the weight w[e]
 // (and w_up[e] in the fused gate/up form); all pointers are device memory.
 struct GroupArgs {
@@ -46,38 +49,50 @@ struct GroupArgs {
     int act;                      // activation of the gate branch in the fused form: 0 = SiLU, 1 = tanh-GELU
     int split_tail;               // dense 128-row DMA form: the last split_tail tiles of every XCD's share go out as two
                                   // half tiles of 64 rows each, to one workgroup apiece
+    int chunk;                    // grouped: column tiles per cell of the tile order (see grouped_tile)
 };
 
-// Which row tile of which group workgroup `b` of a grouped launch works on.  Whole row tiles come first, then
-// the groups' last, partly filled ones: the short tiles fill the gaps at the end of the launch instead of
-// delaying whole tiles queued behind them, and no idle workgroup sits between working ones (workgroups go to
-// the compute units of an XCD in turn: with every other workgroup leaving at once, half of the units idled).
-// The partly filled tiles of a column go to the XCDs (workgroup id % 8) in an order that rotates from column
-// to column: with eight groups each XCD would otherwise work on one group only and the XCD of the group with
-// the most rows would finish last (measured with 10 to 300 rows per group: 9-12 % of the launch).
+// Which row tile of which group, and which column tile, workgroup `b` of a grouped launch works on.
+//
+// The row tiles of all groups form one list: whole row tiles first, then the groups' last, partly filled ones
+// (short tiles then fill the end of the launch instead of delaying whole tiles queued behind them).  Each row tile
+// times `chunk` consecutive column tiles is a cell; the cells, row tile by row tile, are dealt to the 8 XCDs in turn
+// (workgroups go to the XCDs round-robin: XCD = b % 8), and an XCD walks its cells in order, so that
+//   - the workgroups an XCD runs at the same time belong to few row tiles: their rows of x stay in that XCD's L2
+//     (with the column tiles of a row tile spread over all XCDs instead, every XCD read all of x over and over:
+//     the fused gate/up launch of eight groups of 128 rows fetched 1.43 times its weights, and a K step waited
+//     for x to arrive from beyond L2);
+//   - with chunk = ceil(tiles_n / 8) every XCD gets one cell of every row tile: equal shares however uneven the
+//     groups are (a group per XCD was 9-12 % slower with 10 to 300 rows per group);
+//   - with chunk = tiles_n a row tile is one cell: all its column tiles on one XCD, for launches of a single round,
+//     where shares do not matter.
+// Workgroups beyond an XCD's last cell leave at once; they are the last of that XCD's sequence (workgroups go to
+// the compute units of an XCD in turn: idle ones between working ones leave units idle).
 struct GroupTile {
     int group, m0, m_end, tile_n;
 };
 template <int ROWS>
-__device__ inline bool grouped_tile(const int32_t *__restrict__ offsets, int n_groups, int tiles_n, int b, GroupTile &t) {
+__device__ inline bool grouped_tile(const int32_t *__restrict__ offsets, int n_groups, int tiles_n, int chunk, int b,
+                                    GroupTile &t) {
     int full = 0, part = 0;
     for (int e = 0; e < n_groups; e++) {
         const int rows = offsets[e + 1] - offsets[e];
         full += rows / ROWS;
         part += (rows % ROWS) != 0;
     }
-    int idx;
-    bool want_full = true;
-    if (b < full * tiles_n) {
-        idx = b % full;
-        t.tile_n = b / full;
-    } else {
-        b -= full * tiles_n;
-        if (b >= part * tiles_n) return false;
-        want_full = false;
-        t.tile_n = b / part;
-        idx = (b + t.tile_n) % part;
+    const int cells_per_row_tile = (tiles_n + chunk - 1) / chunk, cells = (full + part) * cells_per_row_tile;
+    int i = b >> 3, ci = b & 7, q = 0;
+    for (;; ci += 8) {                                   // this XCD's cells, in order
+        if (ci >= cells) return false;
+        q = ci % cells_per_row_tile;
+        const int size = tiles_n - q * chunk < chunk ? tiles_n - q * chunk : chunk;
+        if (i < size) break;
+        i -= size;
     }
+    t.tile_n = q * chunk + i;
+    int idx = ci / cells_per_row_tile;
+    const bool want_full = idx < full;
+    if (!want_full) idx -= full;
     for (int e = 0; e < n_groups; e++) {
         const int r0 = offsets[e], r1 = offsets[e + 1];
         const int f = (r1 - r0) / ROWS;
@@ -91,7 +106,6 @@ __device__ inline bool grouped_tile(const int32_t *__restrict__ offsets, int n_g
     }
     return false;
 }
-
 // A 64-bit value that is the same in every lane, moved to scalar registers.  (The builtin returns a signed
 // int: each half goes through uint32_t on its way back, or the low half would sign-extend into the high one.)
 __device__ inline uint64_t uniform64(uint64_t v) {
@@ -112,11 +126,14 @@ __device__ inline float gemm_gate_act(float g, int act) {
     return 0.5f * g * (1.0f + t);
 }
 
+
 // GROUPED: the launch covers the row tiles of all groups (see GroupArgs); the tall form then takes one row
 // tile for up to 256 rows of a group and runs only the 32-row blocks that hold rows.
 // DUAL (grouped tall form only): the fused gate/up projection of a gated MLP.  The wave's two 32-row weight
 // blocks are the same 32 rows of the gate and of the up weight (a workgroup covers 128 columns of both), and
-// the epilogue stores act(gate) * up.
+// the epilogue stores act(gate) * up.  With eight waves a wave has one 32-row block: its first tile (16 rows) is
+// the gate's, its second the same 16 rows of the up weight, so that both products of an output element still
+// end in the same lane (accumulator i and i + 8).
 template <int QT, typename AT, bool DMA, int MB, bool GROUPED = false, bool DUAL = false, int WAVES = 4>
 __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                         AT *__restrict__ y, int M, int N, int K, int band_m,
@@ -126,12 +143,12 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     using V8 = typename Vec8<AT>::type;
     static_assert(MB == 4 || (MB == 8 && DMA), "row tiles of 128 rows, or 256 rows in the DMA form");
     static_assert(!DUAL || (GROUPED && MB == 8), "the fused gate/up form exists for grouped launches of the tall form");
-    static_assert(WAVES == 4 || (WAVES == 8 && MB == 8 && DMA && !GROUPED), "eight waves: dense tall form only");
+    static_assert(WAVES == 4 || (WAVES == 8 && MB == 8 && DMA), "eight waves: tall form only");
     constexpr int MB32 = MB, GM = 32 * MB;            // shadow the 128-row constants of the file
     constexpr int NB32 = GN / WAVES / 32;             // 32-row weight blocks per wave: 2, or 1 with eight waves
     // x block of a K step: 8 * MB32 pieces of 1 KiB (layout below), double buffered
-    __shared__ __attribute__((aligned(16))) uint8_t xs0[8 * MB32 * 1024];
-    __shared__ __attribute__((aligned(16))) uint8_t xs1[8 * MB32 * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t xs[2 * 8 * MB32 * 1024];
+    uint8_t *const xs0 = xs, *const xs1 = xs + 8 * MB32 * 1024;
     __shared__ float lut[16];
     if constexpr (QT == QT_NF4) {
         if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODEBOOK[threadIdx.x];
@@ -181,7 +198,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     } else {
         // every workgroup finds its group by walking the offsets (a handful of scalar loads)
         GroupTile gt;
-        if (!grouped_tile<GM>(ga.offsets, ga.n_groups, tn_cnt, blockIdx.x, gt)) return;    // whole workgroup leaves
+        if (!grouped_tile<GM>(ga.offsets, ga.n_groups, tn_cnt, ga.chunk, blockIdx.x, gt)) return;    // whole workgroup leaves
         // (the compiler does not see that what comes out of the walk is the same in every lane)
         tile_n = __builtin_amdgcn_readfirstlane(gt.tile_n);
         m0 = __builtin_amdgcn_readfirstlane(gt.m0);
@@ -190,7 +207,8 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
         w = ga.w[group];
         if constexpr (DUAL) w_up = ga.w_up[group];
     }
-    constexpr int GN_WG = DUAL ? GN / 2 : GN, GN_W = DUAL ? GN_WAVE / 2 : GN / WAVES;   // columns of y per workgroup, per wave
+    constexpr int GN_WG = DUAL ? GN / 2 : GN, GN_W = GN_WG / WAVES;   // columns of y per workgroup, per wave
+    constexpr bool DUAL1 = DUAL && NB32 == 1;     // gate and up rows share the wave's one 32-row block
     const int n0 = tile_n * GN_WG + wave * GN_W;
 
     // weight tiles of this lane: block nb covers rows n0 + 32*nb .. +31 (clamped: a tile row past N
@@ -200,9 +218,11 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     gbytes wt[NB32];
 #pragma unroll
     for (int nb = 0; nb < NB32; nb++) {
-        int trow = n0 / TILE_ROWS + (DUAL ? 0 : nb * 2) + (i32 >> 4);
+        int trow = n0 / TILE_ROWS + (DUAL ? 0 : nb * 2) + (DUAL1 ? 0 : (i32 >> 4));
         trow = trow < n_tiles ? trow : n_tiles - 1;
-        wt[nb] = (gbytes)((DUAL && nb == 1) ? w_up : w) + (int64_t)trow * G * F::TILE_BYTES;
+        const uint8_t *wbase = (DUAL && nb == 1) ? w_up : w;
+        if constexpr (DUAL1) wbase = (i32 >> 4) ? w_up : w;
+        wt[nb] = (gbytes)wbase + (int64_t)trow * G * F::TILE_BYTES;
     }
 
     // The x block of a K step (128 rows x 256 bytes) sits in LDS as 32 pieces of 1 KiB: piece h * 16 + t
@@ -294,15 +314,18 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                      :: "v"(xpiece_off[(MB32 == 8 && !GROUPED) ? j : 0]), "s"(src), "s"(lbase), "n"(j * 1024) : "memory", "m0", "scc");
     };
     // Grouped tall form: a tile holds rows_here <= 256 rows of its group and only the first MBC 32-row blocks are
-    // computed.  Wave w fills the pieces 2j + w % 2 (rows 8 * (2j + w % 2) ..) of half row w / 2 for j < 2 * MBC:
+    // computed.  With HW = WAVES / 2 waves per half row, wave w fills the pieces HW * j + w % HW (rows
+    // 8 * (HW * j + w % HW) ..) of half row w / HW for j < 4 * MBC / HW:
     // the same count for every wave and a bound known at compile time, so that the main loop stays free of
-    // branches.  The two pieces of the last block may reach past the group's rows: they take their rows from a
+    // branches.  The wave's pieces of the last block (two with four waves, one with eight) may reach past the
+    // group's rows: they take their rows from a
     // per-lane offset relative to the tile's first row, with the row clamped to the group's last one (rows past
     // it are computed from a copy of that row and never stored).
+    constexpr unsigned HW = WAVES / 2; constexpr int XPB = 4 / HW;         // waves per half row; pieces per wave and 32-row block
     const int rows_here = __builtin_amdgcn_readfirstlane(M - m0 < GM ? M - m0 : GM);
-    uint64_t xtile_base = (uint64_t)(uintptr_t)x + ((uint64_t)m0 * (uint64_t)K + (uint64_t)(wave >> 1) * 64u) * sizeof(AT);
+    uint64_t xtile_base = (uint64_t)(uintptr_t)x + ((uint64_t)m0 * (uint64_t)K + (uint64_t)((unsigned)wave / HW) * 64u) * sizeof(AT);
     auto tail_offset = [&](int j) __attribute__((always_inline)) {            // piece j of this wave, rows clamped
-        int row = 8 * (2 * j + (wave & 1)) + xr_l[wave & 1];
+        int row = 8 * (int)(HW * j + ((unsigned)wave % HW)) + xr_l[wave & 1];
         row = row < rows_here ? row : rows_here - 1;
         return (uint32_t)row * (uint32_t)K * (uint32_t)sizeof(AT) + (uint32_t)xc_l[wave & 1];
     };
@@ -310,20 +333,36 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     // (voff_tail: this lane's offset from the tile's first row for each of the wave's pieces, the rows of the last
     // block's two clamped; fixed for the walk along K, like the dense forms' - see grouped_piece_offsets below)
     constexpr bool GTALL = GROUPED && MB32 == 8;
-    constexpr int NVOFF = GTALL ? 2 * MB32 : 2;
-    auto dma_x_grouped = [&](int kt, uint8_t *buf, const int j, auto mbc_, const uint32_t (&voff_tail)[NVOFF]) __attribute__((always_inline)) {
-        kt = kt0 + (kt < last ? kt : last);
-        // the same in every lane, which the compiler does not always see after the walk over the groups
-        const uint64_t src = uniform64(xtile_base + (uint64_t)kt * (TILE_COLS * sizeof(AT)));
-        const uint32_t lbase = __builtin_amdgcn_readfirstlane(
-            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + ((wave >> 1) * (4 * MB32) + (wave & 1)) * 1024);
-        asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"(voff_tail[GTALL ? j : 0]), "s"(src), "s"(lbase), "n"(2 * j * 1024) : "memory", "m0", "scc");
+    // Eight waves have half the vector registers: there a wave's pieces share one lane offset (its first piece's)
+    // and the rows of piece j are added to the scalar base; the one piece of the last block keeps its own,
+    // clamped, offset.  (Scalar arithmetic is cheap with two waves per SIMD; with one, every instruction between
+    // two MFMAs is issue time.)
+    constexpr bool SCALAR_ROWS = GTALL && WAVES == 8;
+    constexpr int NVOFF = SCALAR_ROWS ? 2 : GTALL ? XPB * MB32 : 2;
+    // What a variant of the main loop keeps for its LDS-DMAs of x: the lane offsets of the wave's pieces and where
+    // the pieces start within an x buffer (a scalar: the wave index is one)
+    struct XGrouped {
+        uint32_t voff[NVOFF];
+        uint32_t lds_wave_off;
     };
-    auto dma_x = [&](int kt, uint8_t *buf, auto mbc_, const uint32_t (&voff_tail)[NVOFF]) __attribute__((always_inline)) {
+    auto dma_x_grouped = [&](int kt, uint8_t *buf, const int j, auto mbc_, const XGrouped &xg) __attribute__((always_inline)) {
+        constexpr int MBC = decltype(mbc_)::value;
+        const uint32_t (&voff_tail)[NVOFF] = xg.voff;
+        const uint32_t lds_wave_off = xg.lds_wave_off;
+        kt = kt0 + (kt < last ? kt : last);
+        const bool tail = j >= XPB * (MBC - 1);
+        // the same in every lane, which the compiler does not always see after the walk over the groups
+        uint64_t src = xtile_base + (uint64_t)kt * (TILE_COLS * sizeof(AT));
+        if (SCALAR_ROWS && !tail) src += (uint64_t)((uint32_t)(8 * HW * j) * (uint32_t)K * (uint32_t)sizeof(AT));
+        src = uniform64(src);
+        const uint32_t lbase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)buf + lds_wave_off;
+        asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(voff_tail[SCALAR_ROWS ? (tail ? 1 : 0) : GTALL ? j : 0]), "s"(src), "s"(lbase), "n"((int)HW * j * 1024) : "memory", "m0", "scc");
+    };
+    auto dma_x = [&](int kt, uint8_t *buf, auto mbc_, const XGrouped &xg) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < (GTALL ? 2 * decltype(mbc_)::value : PW); j++) {
-            if constexpr (GTALL) dma_x_grouped(kt, buf, j, mbc_, voff_tail);
+        for (int j = 0; j < (GTALL ? XPB * decltype(mbc_)::value : PW); j++) {
+            if constexpr (GTALL) dma_x_grouped(kt, buf, j, mbc_, xg);
             else if constexpr (MB32 == 8) dma_x_scalar(kt, buf, j);
             else dma_x_one(kt, buf, j);
         }
@@ -371,14 +410,14 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     // two waves per SIMD every cycle a wave stands at a memory instruction is a cycle its MFMA pipe idles.
     // `point` = index of the MFMA group (16-column step * row blocks + row block) the call follows.
     auto fetch_units = [&](int kt, uint8_t *buf, WRegs &t, const int point, const int points, auto mbc_,
-                           const uint32_t (&voff_tail)[NVOFF]) __attribute__((always_inline)) {
-        constexpr int UNITS = NB32 + (GTALL ? 2 * decltype(mbc_)::value : PW);
+                           const XGrouped &xg) __attribute__((always_inline)) {
+        constexpr int UNITS = NB32 + (GTALL ? XPB * decltype(mbc_)::value : PW);
         const int spread = points * 5 / 8 > 0 ? points * 5 / 8 : 1;
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             if (u < point * UNITS / spread || u >= (point + 1) * UNITS / spread || point >= spread) continue;
             if (u < NB32) load_w_nb(kt, t, u);
-            else if constexpr (GTALL) dma_x_grouped(kt, buf, u - NB32, mbc_, voff_tail);
+            else if constexpr (GTALL) dma_x_grouped(kt, buf, u - NB32, mbc_, xg);
             else if constexpr (MB32 == 8) dma_x_scalar(kt, buf, u - NB32);
             else dma_x_one(kt, buf, u - NB32);
         }
@@ -387,14 +426,14 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     // The same for the deeper pipeline of the grouped tall form (below): the pieces of x of step kt_x first, then the
     // weight registers of step kt_w, so that the weight loads are the youngest loads in flight when the step ends.
     auto fetch_units_deep = [&](int kt_x, uint8_t *buf, int kt_w, WRegs &t, const int point, const int points, auto mbc_,
-                                const uint32_t (&voff_tail)[NVOFF]) __attribute__((always_inline)) {
-        constexpr int XU = GTALL ? 2 * decltype(mbc_)::value : PW, UNITS = XU + NB32;
+                                const XGrouped &xg) __attribute__((always_inline)) {
+        constexpr int XU = GTALL ? XPB * decltype(mbc_)::value : PW, UNITS = XU + NB32;
         const int spread = points * 5 / 8 > 0 ? points * 5 / 8 : 1;
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             if (u < point * UNITS / spread || u >= (point + 1) * UNITS / spread || point >= spread) continue;
             if (u < XU) {
-                if constexpr (GTALL) dma_x_grouped(kt_x, buf, u, mbc_, voff_tail);
+                if constexpr (GTALL) dma_x_grouped(kt_x, buf, u, mbc_, xg);
                 else if constexpr (MB32 == 8) dma_x_scalar(kt_x, buf, u);
                 else dma_x_one(kt_x, buf, u);
             }
@@ -440,6 +479,10 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     auto compute = [&](auto &acc, const uint8_t *cur, const WRegs &t, auto mbc_, auto &&between) __attribute__((always_inline)) {
         constexpr int MBC = decltype(mbc_)::value;
         constexpr int SLOTS = MBC * NB32, PAIRS = 4 * NB32;   // MFMAs per 16-column step; register pairs to dequantize meanwhile
+        // MFMA slots that carry the dequantization of the next 16-column step.  A wave with one weight block uses
+        // what it dequantizes in the very next MFMA after the step's last one: that last slot then stays empty,
+        // so that a whole MFMA lies between the last write of an operand and its use.
+        constexpr int SPREAD = (NB32 == 1 && SLOTS > 1) ? SLOTS - 1 : SLOTS;
         V8 xv[MBC];
         u32x4 wv[NB32];
 #pragma unroll
@@ -463,7 +506,10 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
             for (int mb = 0; mb < MBC; mb++) {
 #pragma unroll
                 for (int nb = 0; nb < NB32; nb++) {
-                    mfma_acc<WAIT_STATES>(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    // (a wave with one weight block uses what the step before dequantized last in the very first MFMA of a
+                    // step, and where the compiler puts that last instruction is its choice: the two wait states stay)
+                    if (NB32 == 1 && mb == 0) mfma_acc<true>(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    else mfma_acc<WAIT_STATES>(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
                     if (ks < 7) {
                         // pairs [ceil(slot * PAIRS / SLOTS), ceil((slot + 1) * PAIRS / SLOTS)): spread evenly over the
                         // MFMA slots, the first slot of a row block served first (the second is followed by the LDS
@@ -471,7 +517,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                         const int slot_i = mb * NB32 + nb;
 #pragma unroll
                         for (int idx = 0; idx < PAIRS; idx++) {
-                            if (idx < (slot_i * PAIRS + SLOTS - 1) / SLOTS || idx >= ((slot_i + 1) * PAIRS + SLOTS - 1) / SLOTS) continue;
+                            if (slot_i >= SPREAD || idx < (slot_i * PAIRS + SPREAD - 1) / SPREAD || idx >= ((slot_i + 1) * PAIRS + SPREAD - 1) / SPREAD) continue;
                             wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);   // (weight block, pair)
                         }
                     }
@@ -525,9 +571,11 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
         constexpr int MBC = decltype(mbc_)::value;
         constexpr bool HAS_NEXT = true;
         constexpr int SLOTS = MBC * NB32, PAIRS = 4 * NB32;
+        constexpr int SPREAD = (NB32 == 1 && SLOTS > 1) ? SLOTS - 1 : SLOTS;     // (see compute)
         constexpr bool WAIT_STATES = SLOTS < 4;          // (see compute)
         constexpr int BMB = MBC > 2 ? 1 : 0;
         constexpr int TAIL = (MBC - 1 - BMB) * NB32;     // MFMA slots of the last 16-column step behind the barrier
+        constexpr int TSPREAD = (NB32 == 1 && TAIL > 1) ? TAIL - 1 : TAIL;      // of them, those that carry dequantization
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
             u32x4 wn[NB32];
@@ -535,12 +583,15 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
             for (int mb = 0; mb < MBC; mb++) {
 #pragma unroll
                 for (int nb = 0; nb < NB32; nb++) {
-                    mfma_acc<WAIT_STATES>(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    // (a wave with one weight block uses what the step before dequantized last in the very first MFMA of a
+                    // step, and where the compiler puts that last instruction is its choice: the two wait states stay)
+                    if (NB32 == 1 && mb == 0) mfma_acc<true>(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
+                    else mfma_acc<WAIT_STATES>(acc[mb][nb], __builtin_bit_cast(V8, wv[nb]), xv[mb]);
                     if (ks < 7) {
                         const int slot_i = mb * NB32 + nb;
 #pragma unroll
                         for (int idx = 0; idx < PAIRS; idx++) {
-                            if (idx < (slot_i * PAIRS + SLOTS - 1) / SLOTS || idx >= ((slot_i + 1) * PAIRS + SLOTS - 1) / SLOTS) continue;
+                            if (slot_i >= SPREAD || idx < (slot_i * PAIRS + SPREAD - 1) / SPREAD || idx >= ((slot_i + 1) * PAIRS + SPREAD - 1) / SPREAD) continue;
                             wn[idx >> 2][idx & 3] = dequant_pair(t, ks + 1, idx >> 2, idx & 3);
                         }
                     } else if constexpr (HAS_NEXT && TAIL > 0) {
@@ -548,7 +599,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                             const int ts = (mb - BMB - 1) * NB32 + nb;
 #pragma unroll
                             for (int idx = 0; idx < PAIRS; idx++) {
-                                if (idx < (ts * PAIRS + TAIL - 1) / TAIL || idx >= ((ts + 1) * PAIRS + TAIL - 1) / TAIL) continue;
+                                if (ts >= TSPREAD || idx < (ts * PAIRS + TSPREAD - 1) / TSPREAD || idx >= ((ts + 1) * PAIRS + TSPREAD - 1) / TSPREAD) continue;
                                 wn[idx >> 2][idx & 3] = dequant_pair(tn, 0, idx >> 2, idx & 3);
                             }
                         }
@@ -611,7 +662,8 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     constexpr int CH = GN_W * (int)sizeof(AT) / 16;          // 16-byte chunks per row of this wave's columns
     constexpr int REGION = GM * CH * 16;                     // bytes per wave: WAVES / 2 of them fit an x buffer
     static_assert(REGION * (WAVES / 2) <= 8 * MB32 * 1024, "a wave's rows fit its share of an x buffer");
-    static_assert(CH == (DUAL ? 4 : NB32 * 4), "one chunk per group of four accumulator registers and kg pair");
+    static_assert(CH == (DUAL1 ? 2 : DUAL ? 4 : NB32 * 4), "one chunk per group of four accumulator registers and kg pair");
+    constexpr int QN = DUAL1 ? 2 : 4;                        // register groups of a block that hold columns of y
     if constexpr (!DUAL) {
         if (ws) {
             // Partial sums of a K split keep the register layout (split, tile, wave, register group, lane): every
@@ -650,14 +702,16 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
             for (int nb = 0; nb < (DUAL ? 1 : NB32); nb++) {
                 // (keeps the block in its accumulation registers up to here: the compiler would otherwise read
                 // all blocks into vector registers ahead of the branch that picks this form of the epilogue)
-                if constexpr (DUAL) asm volatile("" : "+a"(acc[mb][0]), "+a"(acc[mb][1]));
+                if constexpr (DUAL && !DUAL1) asm volatile("" : "+a"(acc[mb][0]), "+a"(acc[mb][1]));
                 else asm volatile("" : "+a"(acc[mb][nb]));
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
+                for (int q = 0; q < QN; q++) {
                     at4 o;
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        if constexpr (DUAL) o[i] = to_at<AT>(gemm_gate_act(acc[mb][0][q * 4 + i], ga.act) * acc[mb][1][q * 4 + i]);
+                        // (one block for both: registers 0..7 hold the gate's 16 rows, 8..15 the up weight's)
+                        if constexpr (DUAL1) o[i] = to_at<AT>(gemm_gate_act(acc[mb][0][q * 4 + i], ga.act) * acc[mb][0][8 + q * 4 + i]);
+                        else if constexpr (DUAL) o[i] = to_at<AT>(gemm_gate_act(acc[mb][0][q * 4 + i], ga.act) * acc[mb][1][q * 4 + i]);
                         else o[i] = to_at<AT>(acc[mb][nb][q * 4 + i]);
                     }
                     *(at4 *)(wpos[nb * 4 + q] + mb * 32 * (CH * 16)) = o;
@@ -691,17 +745,19 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
         const int m = m0 + mb * 32 + i32;
         if constexpr (DUAL) {
             // both blocks hold the same 32 columns of y: the gate branch in block 0, the up branch in block 1
-            asm volatile("" : "+a"(acc[mb][0]), "+a"(acc[mb][1]));     // (stay in accumulation registers up to here)
+            if constexpr (DUAL1) asm volatile("" : "+a"(acc[mb][0]));
+            else asm volatile("" : "+a"(acc[mb][0]), "+a"(acc[mb][NB32 - 1]));     // (stay in accumulation registers up to here)
             if (m < M) {
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
+                for (int q = 0; q < QN; q++) {
                     const int n = n0 + q * 8 + kg * 4;
                     if (n < N) {
                         typedef AT at4 __attribute__((ext_vector_type(4)));
                         at4 o;
 #pragma unroll
                         for (int i = 0; i < 4; i++)
-                            o[i] = to_at<AT>(gemm_gate_act(acc[mb][0][q * 4 + i], ga.act) * acc[mb][1][q * 4 + i]);
+                            o[i] = to_at<AT>(gemm_gate_act(acc[mb][0][q * 4 + i], ga.act) *
+                                             (DUAL1 ? acc[mb][0][8 + q * 4 + i] : acc[mb][NB32 - 1][q * 4 + i]));
                         *(at4 *)(y + (int64_t)m * N + n) = o;
                     }
                 }
@@ -748,14 +804,21 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                 uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(xtile_base >> 32));
                 asm volatile("" : "+s"(lo), "+s"(hi));
                 xtile_base = (uint64_t)lo | ((uint64_t)hi << 32);
-                asm volatile("" : "+v"(wt[0]), "+v"(wt[1]));
+                if constexpr (NB32 == 2) asm volatile("" : "+v"(wt[0]), "+v"(wt[1]));
+                else asm volatile("" : "+v"(wt[0]));
             }
-            uint32_t voff_tail[NVOFF] = {};               // grouped_piece_offsets
-            if constexpr (GTALL) {
+            XGrouped xg = {};                             // grouped_piece_offsets
+            uint32_t (&voff_tail)[NVOFF] = xg.voff;
+            xg.lds_wave_off = (uint32_t)__builtin_amdgcn_readfirstlane(
+                (int)((((unsigned)wave / HW) * (4 * MB32) + ((unsigned)wave % HW)) * 1024));
+            if constexpr (SCALAR_ROWS) {
+                voff_tail[0] = xlane_off_wave + (uint32_t)(8 * ((unsigned)wave % HW)) * (uint32_t)K * (uint32_t)sizeof(AT);
+                voff_tail[1] = tail_offset(XPB * (MBC - 1));
+            } else if constexpr (GTALL) {
 #pragma unroll
-                for (int j = 0; j < 2 * MBC; j++)
-                    voff_tail[j] = j >= 2 * (MBC - 1) ? tail_offset(j)
-                                                       : xlane_off_wave + (uint32_t)(8 * (2 * j + (wave & 1))) * (uint32_t)K * (uint32_t)sizeof(AT);
+                for (int j = 0; j < XPB * MBC; j++)
+                    voff_tail[j] = j >= XPB * (MBC - 1) ? tail_offset(j)
+                                                         : xlane_off_wave + (uint32_t)(8 * (HW * j + ((unsigned)wave % HW))) * (uint32_t)K * (uint32_t)sizeof(AT);
             }
             if constexpr (GTALL && MBC < 8) {
                 // Tiles of a few row blocks have short K steps: with one step of prefetch a step lasted as long as
@@ -766,7 +829,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                 // one step of prefetch (it comes from L2).  Three weight sets and two buffers: a period of six.
                 constexpr int WLOADS = NB32 * ((F::BITS == 8 ? 2 : 1) * 2 + 1);      // load instructions of load_w_nb, all blocks
                 WRegs w2;
-                dma_x(0, xs0, mbc, voff_tail);
+                dma_x(0, xs0, mbc, xg);
                 load_w(0, w0);
                 load_w(1, w1);
                 wait_all_loads();
@@ -774,7 +837,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
 #define LOWBIT_DEEP_STEP(i, cur, nxt, wc, wl)                                                                  \
                 if (kt + (i) < Gs) {                                                                           \
                     compute(acc, cur, wc, mbc, [&](const int point, const int points) __attribute__((always_inline)) { \
-                        fetch_units_deep(kt + (i) + 1, nxt, kt + (i) + 2, wl, point, points, mbc, voff_tail); \
+                        fetch_units_deep(kt + (i) + 1, nxt, kt + (i) + 2, wl, point, points, mbc, xg); \
                     });                                                                                        \
                     wait_loads_but<WLOADS>();                                                                  \
                     __syncthreads();                                                                           \
@@ -792,7 +855,7 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
                 epilogue(acc, mbc);
                 return;
             }
-            dma_x(0, xs0, mbc, voff_tail);
+            dma_x(0, xs0, mbc, xg);
             load_w(0, w0);
             wait_all_loads();
             __syncthreads();
@@ -802,10 +865,10 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
             first_operands(xs0, w0, mbc, xv, wv);
             for (int kt = 0; kt + 1 < Gs; kt += 2) {
                 step_ahead(acc, xs0, xs1, w0, w1, mbc, xv, wv, [&](const int point, const int points) __attribute__((always_inline)) {
-                    fetch_units(kt + 1, xs1, w1, point, points, mbc, voff_tail);
+                    fetch_units(kt + 1, xs1, w1, point, points, mbc, xg);
                 });
                 step_ahead(acc, xs1, xs0, w1, w0, mbc, xv, wv, [&](const int point, const int points) __attribute__((always_inline)) {   // past the end: clamped, unused re-reads
-                    fetch_units(kt + 2, xs0, w0, point, points, mbc, voff_tail);
+                    fetch_units(kt + 2, xs0, w0, point, points, mbc, xg);
                 });
             }
             if (Gs & 1) step_ahead(acc, xs0, xs1, w0, w1, mbc, xv, wv, nothing);

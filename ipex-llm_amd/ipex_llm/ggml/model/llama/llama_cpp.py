@@ -289,6 +289,18 @@ def lowbit_grouped_workspace_bytes(n_groups, total_rows, n, k):
     return int(_lib.lowbit_grouped_workspace_bytes(n_groups, total_rows, n, k))
 
 
+_lib.lowbit_grouped_forward_plan.argtypes = [c_int, c_int64, c_int64, c_int64, c_int, c_size_t, ctypes.POINTER(c_int)]
+_lib.lowbit_grouped_forward_plan.restype = c_int
+
+
+def lowbit_grouped_forward_plan(n_groups, total_rows, n, k, have_workspace, workspace_bytes=0):
+    """(tall, splits, waves, workgroups per split) of a plain grouped product; host arithmetic only."""
+    out = (c_int * 4)()
+    _check(_lib.lowbit_grouped_forward_plan(n_groups, total_rows, n, k, int(bool(have_workspace)), workspace_bytes, out),
+           "lowbit_grouped_forward_plan")
+    return tuple(out)
+
+
 def lowbit_grouped_forward_ws(x, w_ptrs, y, group_offsets, n_groups, total_rows, qtype, act_dtype, n, k, workspace,
                               workspace_bytes, stream):
     _check(_lib.lowbit_grouped_forward_ws(x, w_ptrs, y, group_offsets, n_groups, total_rows, qtype, act_dtype,

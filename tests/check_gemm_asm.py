@@ -13,13 +13,20 @@ compiler went along with it, per kernel of an assembly listing (hipcc -S --cuda-
      loses a K step for the block written last;
   2. no such register is overwritten (v_accvgpr_mov, v_accvgpr_write) that soon after its MFMA either;
   3. the kernel uses no scratch memory and calls no function (a variant of the main loop that is not inlined
-     keeps its closure in scratch and reads the weights with flat loads);
+     keeps its closure in scratch and reads the weights with flat loads); kernels named after --allow-scratch may
+     spill anywhere, kernels named after --allow-scratch-outside-loops only outside loops that hold MFMAs;
   4. no LDS-DMA takes its scalar base address from a v_readfirstlane less than 5 wait states earlier (VALU
      write of an SGPR followed by a VMEM read of it);
   5. no MFMA reads a vector register as its A or B operand that a VALU instruction wrote less than 2 wait states
-     earlier (the kernels leave the wait states out where the operands are ready long before).
+     earlier (the kernels leave the wait states out where the operands are ready long before);
+  6. a wait that leaves N loads in flight ahead of a workgroup barrier ("s_waitcnt vmcnt(N)", N > 0, then s_barrier:
+     the step of the deep pipeline, whose youngest loads are the weights of two steps ahead) has at least N load
+     instructions between the last LDS-DMA ahead of it and itself - loads retire in order, so with fewer (the
+     compiler merged or dropped one) an LDS-DMA of x could still be in flight when the barrier publishes its buffer.
+     A wait that the source marks with the comment "lowbit: this wait keeps the loads of one step in flight"
+     (x two steps ahead as well) needs that many loads, LDS-DMAs included, since the barrier ahead of it.
 
-usage: check_gemm_asm.py listing.s [--allow-scratch SUBSTRING ...]
+usage: check_gemm_asm.py listing.s [--allow-scratch SUBSTRING ...] [--allow-scratch-outside-loops SUBSTRING ...]
 Exit status 0 when every kernel passes, 1 otherwise.
 """
 import re
@@ -63,9 +70,35 @@ def vregs(spec):
     return {int(m.group(1))} if m else set()
 
 
-def check_kernel(name, lines, allow_scratch, first_line=0):
+def mfma_loops(lines):
+    """Line numbers that lie inside a loop holding an MFMA, from the loop comments the compiler puts behind block
+    labels ('=>This Inner Loop Header', 'in Loop: Header=BB1_23', also on the '; %bb.N:' lines of blocks that
+    are fallen into)."""
+    loop_of = {}                                   # line -> header name of the innermost loop it is in
+    current = None
+    for no, line in enumerate(lines):
+        t = line.strip()
+        m = re.match(r"(?:\.L(BB\w+):|; %bb\.\d+:)(.*)", t)
+        if m:
+            rest = m.group(2)
+            h = re.search(r"Header=(BB\w+)", rest)
+            if "Loop Header" in rest and m.group(1):
+                current = m.group(1)
+            elif h:
+                current = h.group(1)
+            else:
+                current = None
+        if current:
+            loop_of[no] = current
+    with_mfma = {h for no, h in loop_of.items() if "v_mfma" in lines[no]}
+    return {no for no, h in loop_of.items() if h in with_mfma}
+
+
+def check_kernel(name, lines, allow_scratch, first_line=0, allow_outside_loops=()):
     errors = []
     ins = [(no + first_line, t) for no, t in instructions(lines)]
+    in_mfma_loop = {no + first_line for no in mfma_loops(lines)}
+    scratch_seen = False
     mfma_dst = set()
     mfma_at = []
     for k, (no, t) in enumerate(ins):
@@ -118,8 +151,11 @@ def check_kernel(name, lines, allow_scratch, first_line=0):
         if re.match(r"s_swappc_b64|s_call_b64", t):
             errors.append(f"line {no + 1}: function call: {t}")
         if t.startswith("scratch_") and not any(a in name for a in allow_scratch):
-            errors.append(f"line {no + 1}: scratch access: {t}")
-            break
+            in_loop = no in in_mfma_loop
+            if in_loop or not any(a in name for a in allow_outside_loops):
+                if not scratch_seen or in_loop:
+                    errors.append(f"line {no + 1}: scratch access{' inside an MFMA loop' if in_loop else ''}: {t}")
+                scratch_seen = True
         m = re.match(r"v_mfma_\S+ a\[\d+:\d+\], (v\[\d+:\d+\]), (v\[\d+:\d+\])", t)
         if m:
             src = vregs(m.group(1)) | vregs(m.group(2))
@@ -134,6 +170,26 @@ def check_kernel(name, lines, allow_scratch, first_line=0):
                 w += wait_states(tj)
                 if w >= 2 or re.match(r"s_branch|s_cbranch|s_endpgm|s_setpc_b64", tj):
                     break
+        m = re.match(r"s_waitcnt vmcnt\((\d+)\)$", t)
+        if m and int(m.group(1)) > 0 and any(ins[j][1].startswith("s_barrier") for j in range(k + 1, min(k + 4, len(ins)))):
+            whole_step = any("lowbit: this wait keeps the loads of one step in flight" in l
+                             for l in lines[max(0, no - first_line - 8):no - first_line])
+            younger, found = 0, False
+            for j in range(k - 1, -1, -1):
+                tj = ins[j][1]
+                if tj.startswith("global_load_lds") and not whole_step:
+                    found = True
+                    break
+                if re.match(r"(?:global|flat|scratch|buffer)_load", tj):
+                    younger += 1
+                if tj.startswith("s_barrier") and whole_step:
+                    found = True
+                    break
+                if re.match(r"s_branch|s_cbranch|s_endpgm|s_setpc_b64|s_barrier", tj):
+                    break
+            if found and younger < int(m.group(1)):
+                errors.append(f"line {no + 1}: {t} ahead of a barrier with only {younger} loads "
+                              + ("since the barrier before it" if whole_step else "behind the last LDS-DMA"))
         m = re.match(r"global_load_lds_dwordx4 v\d+, s\[(\d+):(\d+)\]", t)
         if m:
             base = {int(m.group(1)), int(m.group(2))}
@@ -153,7 +209,11 @@ def main(argv):
     if len(argv) < 2:
         print(__doc__)
         return 2
-    allow = []
+    allow, allow_outside = [], []
+    if "--allow-scratch-outside-loops" in argv:
+        i = argv.index("--allow-scratch-outside-loops")
+        allow_outside = argv[i + 1:]
+        argv = argv[:i]
     if "--allow-scratch" in argv:
         i = argv.index("--allow-scratch")
         allow = argv[i + 1:]
@@ -166,7 +226,7 @@ def main(argv):
         if "gemm_mfma_kernel" not in name and "gemm_ring_kernel" not in name:
             continue
         e = starts[n + 1] if n + 1 < len(starts) else len(text)
-        errors = check_kernel(name, text[s:e], allow, s)
+        errors = check_kernel(name, text[s:e], allow, s, allow_outside)
         label = "ok" if not errors else f"{len(errors)} problem(s)"
         print(f"{name}: {label}")
         for msg in errors[:10]:

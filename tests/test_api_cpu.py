@@ -3,6 +3,8 @@ import ctypes
 import os
 import re
 
+import numpy as np
+
 import pytest
 import torch
 from torch import nn
@@ -409,3 +411,25 @@ def test_fused_experts_module_is_replaced_expert_by_expert():
         m2 = nn.Sequential(Block(192, 256)).eval()
     m2, _ = _replace_with_low_bit_linear(m2, Q["fp8_e4m3"], convert_shape_only=True)
     assert isinstance(m2[0].experts, _FusedExperts)
+
+
+def test_grouped_split_workspace_holds_a_tile_for_every_workgroup():
+    """Every workgroup of a K-split grouped launch writes one 256 x 256 fp32 tile at its own index: the workspace
+    the library asks for must hold splits x workgroups of them, whatever tile order the launch takes (a grid that
+    grew with the tile order once overran a workspace sized from the tile count).  Host arithmetic only."""
+    rng = np.random.default_rng(11)
+    tile = 256 * 256 * 4
+    shapes = [(12, 1917, 272, 2048), (8, 1024, 4096, 14336), (8, 1024, 14336, 4096), (8, 256, 4096, 14336), (1, 40, 512, 8192)]
+    shapes += [(int(rng.integers(1, 70)), int(rng.integers(1, 5000)), 16 * int(rng.integers(1, 1200)), 128 * int(rng.integers(1, 120)))
+               for _ in range(300)]
+    split_seen = False
+    for n_groups, rows, n, k in shapes:
+        need = ggml.lowbit_grouped_workspace_bytes(n_groups, rows, n, k)
+        for ws in {need, need // 2, 0}:
+            tall, splits, waves, grid = ggml.lowbit_grouped_forward_plan(n_groups, rows, n, k, ws > 0, ws)
+            assert splits >= 1 and waves in (4, 8) and grid % 8 == 0 and grid >= 8
+            if splits > 1:
+                split_seen = True
+                assert tall == 1 and splits * grid * tile <= ws, (n_groups, rows, n, k, ws, splits, grid)
+        assert (need == 0) == (ggml.lowbit_grouped_forward_plan(n_groups, rows, n, k, True, 1 << 40)[1] == 1)
+    assert split_seen

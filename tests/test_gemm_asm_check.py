@@ -1,5 +1,5 @@
 """The MFMA GEMM kernels keep their MFMAs in inline assembly, which hides from the compiler that accumulator
-blocks are still in flight after them.  ipex-llm_amd/csrc/check_gemm_asm.py looks through the generated assembly
+blocks are still in flight after them.  tests/check_gemm_asm.py looks through the generated assembly
 for what that can break (accumulator blocks copied or read too early, scratch memory, function calls, scalar
 base addresses written by the vector unit right ahead of an LDS-DMA, MFMA operands written by the vector unit
 right ahead of the MFMA).  Here it runs on every GEMM translation unit - the grouped formats, the dense GEMM, the
@@ -13,6 +13,7 @@ import sys
 import pytest
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ipex-llm_amd", "csrc")
+CHECKER = os.path.join(os.path.dirname(os.path.abspath(__file__)), "check_gemm_asm.py")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
          "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-fast-math", "-Xclang", "-target-feature", "-Xclang",
@@ -40,8 +41,10 @@ def listings(tmp_path_factory):
 def test_generated_assembly_respects_the_mfma_hazards(unit, listings):
     listing = listings[unit]
     assert isinstance(listing, str), "hipcc failed on %s with code %s" % (unit, listing)
-    # the 128-row DMA form is held to 128 vector registers, for two workgroups per compute unit, and spills a few
-    out = subprocess.run([sys.executable, os.path.join(CSRC, "check_gemm_asm.py"), listing, "--allow-scratch", "Lb1ELi4E"],
+    # the 128-row DMA form is held to 128 vector registers, for two workgroups per compute unit, and spills a few;
+    # the grouped tall form with eight waves (two per SIMD, 128 vector registers each) may spill outside its loops
+    out = subprocess.run([sys.executable, CHECKER, listing, "--allow-scratch", "Lb1ELi4E",
+                          "--allow-scratch-outside-loops", "Li8ELb1ELb1ELi8E"],
                          capture_output=True, text=True)
     assert out.returncode == 0, out.stdout[-4000:]
     assert out.stdout.count(": ok") >= 3, out.stdout
@@ -57,7 +60,7 @@ def test_the_checker_sees_a_copy_of_a_fresh_accumulator(tmp_path):
                    "\tv_accvgpr_mov_b32 a40, a0\n"          # written two MFMAs ago: fine
                    "\tv_accvgpr_mov_b32 a41, a16\n"         # written by the MFMA just issued: not fine
                    "\ts_endpgm\n")
-    out = subprocess.run([sys.executable, os.path.join(CSRC, "check_gemm_asm.py"), str(bad)], capture_output=True, text=True)
+    out = subprocess.run([sys.executable, CHECKER, str(bad)], capture_output=True, text=True)
     assert out.returncode == 1
     assert "a41, a16" in out.stdout and "a40, a0" not in out.stdout
 
@@ -75,6 +78,60 @@ def test_the_checker_sees_an_mfma_operand_written_right_ahead_of_it(tmp_path):
                    "\tv_mfma_f32_32x32x16_f16 a[32:47], v[8:11], v[4:7], a[32:47]\n"   # writes another register: fine
                    "\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n"
                    "\ts_endpgm\n")
-    out = subprocess.run([sys.executable, os.path.join(CSRC, "check_gemm_asm.py"), str(bad)], capture_output=True, text=True)
+    out = subprocess.run([sys.executable, CHECKER, str(bad)], capture_output=True, text=True)
     assert out.returncode == 1
     assert out.stdout.count("MFMA operand written by VALU") == 1 and "v9, v20, v21" in out.stdout
+
+
+def test_the_checker_keeps_checking_after_a_spill_and_tells_loops_from_straight_code(tmp_path):
+    """A spill used to end the check of a kernel: an operand hazard behind it went unseen.  Spills outside loops
+    can be allowed per kernel; inside a loop that holds MFMAs they never are."""
+    text = ("_Z16gemm_mfma_kernelILi8ELb1ELb0ELi8EEv:\n"
+            "\tscratch_store_dword off, v1, off\n"                 # outside any loop
+            ".LBB0_1:                                ; =>This Inner Loop Header: Depth=1\n"
+            "\tscratch_load_dword v1, off, off\n"                   # inside the MFMA loop
+            "\tv_pk_mul_f16 v3, v20, v21\n"
+            "\tv_mfma_f32_32x32x16_f16 a[0:15], v[0:3], v[4:7], a[0:15]\n"
+            "\ts_cbranch_scc1 .LBB0_1\n"
+            "; %bb.2:\n"
+            "\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n"
+            "\tscratch_load_dword v2, off, off\n"                   # behind the loop
+            "\ts_endpgm\n")
+    bad = tmp_path / "bad3.s"
+    bad.write_text(text)
+    out = subprocess.run([sys.executable, CHECKER, str(bad), "--allow-scratch-outside-loops", "Li8ELb1ELb0ELi8E"],
+                         capture_output=True, text=True)
+    assert out.returncode == 1
+    assert out.stdout.count("scratch access") == 1 and "inside an MFMA loop" in out.stdout
+    assert out.stdout.count("MFMA operand written by VALU") == 1
+    out = subprocess.run([sys.executable, CHECKER, str(bad)], capture_output=True, text=True)
+    assert "scratch access:" in out.stdout and "inside an MFMA loop" in out.stdout      # nothing allowed: both kinds
+
+
+def test_the_checker_counts_the_loads_behind_the_last_lds_dma_of_a_deep_step(tmp_path):
+    body = ("_Z16gemm_mfma_kernelv:\n"
+            "\tglobal_load_lds_dwordx4 v1, s[0:1]\n"
+            "%s"
+            "\tv_mfma_f32_32x32x16_f16 a[0:15], v[0:3], v[4:7], a[0:15]\n"
+            "\ts_waitcnt vmcnt(3)\n"
+            "\ts_barrier\n"
+            "\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n"
+            "\ts_endpgm\n")
+    load = "\tglobal_load_dwordx4 v[8:11], v[20:21], off\n"
+    for n_loads, rc in ((3, 0), (2, 1)):
+        f = tmp_path / ("deep%d.s" % n_loads)
+        f.write_text(body % (load * n_loads))
+        out = subprocess.run([sys.executable, CHECKER, str(f)], capture_output=True, text=True)
+        assert out.returncode == rc, out.stdout
+        assert ("behind the last LDS-DMA" in out.stdout) == bool(rc)
+    # x two steps ahead as well: the marked wait leaves a whole step's loads in flight, LDS-DMAs included
+    step = ("\ts_barrier\n" + "\tglobal_load_lds_dwordx4 v1, s[0:1]\n" * 2 + "%s"
+            "\t;;#ASMSTART\n\t; lowbit: this wait keeps the loads of one step in flight\n\t;;#ASMEND\n"
+            "\ts_waitcnt vmcnt(4)\n\ts_barrier\n")
+    for n_loads, rc in ((2, 0), (1, 1)):
+        f = tmp_path / ("deep2_%d.s" % n_loads)
+        f.write_text("_Z16gemm_mfma_kernelv:\n\tv_mfma_f32_32x32x16_f16 a[0:15], v[0:3], v[4:7], a[0:15]\n"
+                     + step % (load * n_loads) + "\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_endpgm\n")
+        out = subprocess.run([sys.executable, CHECKER, str(f)], capture_output=True, text=True)
+        assert out.returncode == rc, out.stdout
+        assert ("since the barrier before it" in out.stdout) == bool(rc)

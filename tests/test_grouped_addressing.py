@@ -11,19 +11,29 @@ import pytest
 ROWS = 256
 
 
-def grouped_tile(offs, tiles_n, b):
+def grouped_tile(offs, tiles_n, chunk, b):
+    """Cells of `chunk` column tiles of one row tile, dealt to the XCDs (b % 8) in turn; an XCD walks its cells in
+    order.  Whole row tiles first, then the groups' partly filled ones."""
     n = len(offs) - 1
     full = sum((offs[e + 1] - offs[e]) // ROWS for e in range(n))
     part = sum(((offs[e + 1] - offs[e]) % ROWS) != 0 for e in range(n))
-    want_full = True
-    if b < full * tiles_n:
-        idx, tn = b % full, b // full
-    else:
-        b -= full * tiles_n
-        if b >= part * tiles_n:
+    per_row_tile = (tiles_n + chunk - 1) // chunk
+    cells = (full + part) * per_row_tile
+    i, ci = b >> 3, b & 7
+    while True:
+        if ci >= cells:
             return None
-        want_full, tn = False, b // part
-        idx = (b + tn) % part             # groups rotate over the XCDs (workgroup id % 8) from column to column
+        q = ci % per_row_tile
+        size = min(chunk, tiles_n - q * chunk)
+        if i < size:
+            break
+        i -= size
+        ci += 8
+    tn = q * chunk + i
+    idx = ci // per_row_tile
+    want_full = idx < full
+    if not want_full:
+        idx -= full
     for e in range(n):
         r0, r1 = offs[e], offs[e + 1]
         f = (r1 - r0) // ROWS
@@ -36,6 +46,11 @@ def grouped_tile(offs, tiles_n, b):
                 return e, r0 + f * ROWS, r1, tn
             idx -= 1
     return None
+
+
+def grouped_grid(row_tiles, tiles_n, chunk):
+    cells = row_tiles * ((tiles_n + chunk - 1) // chunk)
+    return 8 * ((cells + 7) // 8) * chunk
 
 
 def lane_row_chunk(lane, parity):
@@ -53,31 +68,37 @@ def operand_offset(lane, t):
     return p * 1024 + ((r ^ (p & 1)) * 8 + ((2 * t + kg) ^ r)) * 16
 
 
-def check(counts, k, tiles_n=3):
+def check(counts, k, tiles_n=3, chunk=None, waves=4):
     offs = [0] + [int(v) for v in np.cumsum(counts)]
     total = offs[-1]
-    n_wg = tiles_n * (total // ROWS + len(counts))
+    chunk = chunk or (tiles_n + 7) // 8
+    n_wg = grouped_grid(total // ROWS + len(counts), tiles_n, chunk)
     x_bytes = total * k * 2
     seen = set()
+    hw = waves // 2                                # waves per half row
+    idle_seen = [False] * 8
     for b in range(n_wg):
-        t = grouped_tile(offs, tiles_n, b)
+        t = grouped_tile(offs, tiles_n, chunk, b)
         if t is None:
+            idle_seen[b & 7] = True
             continue
+        assert not idle_seen[b & 7], "an idle workgroup ahead of a working one on the same XCD"
         e, m0, m_end, tn = t
         assert (e, m0, tn) not in seen
         seen.add((e, m0, tn))
         assert offs[e] <= m0 < m_end <= offs[e + 1] and (m0 - offs[e]) % ROWS == 0
         rows_here = min(m_end - m0, ROWS)
         mbc = min((m_end - m0 + 31) // 32, 8)
+        half_row = 32                                # pieces per half row of an x buffer
         lds = {}                                  # 16-byte slot -> (row of the tile, byte column of the K step) it holds
-        for wave in range(4):
-            h = wave >> 1
+        for wave in range(waves):
+            h = wave // hw
             tile_base = (m0 * k + h * 64) * 2
-            for j in range(2 * mbc):
-                tail = j >= 2 * (mbc - 1)
-                piece_row = 8 * (2 * j + (wave & 1))
-                piece = h * 32 + 2 * j + (wave & 1)
-                assert piece < 64
+            for j in range(4 // hw * mbc):
+                tail = j >= 4 // hw * (mbc - 1)
+                piece_row = 8 * (hw * j + wave % hw)
+                piece = h * half_row + hw * j + wave % hw
+                assert piece % 2 == wave & 1 and piece < 2 * half_row
                 for lane in range(64):
                     r, c = lane_row_chunk(lane, wave & 1)
                     if tail:
@@ -97,7 +118,7 @@ def check(counts, k, tiles_n=3):
             for mb in range(mbc):
                 for lane in range(64):
                     kg, i32 = lane >> 5, lane & 31
-                    slot = ((ks // 4) * 32 + 4 * mb) * 1024 + operand_offset(lane, ks % 4)
+                    slot = ((ks // 4) * half_row + 4 * mb) * 1024 + operand_offset(lane, ks % 4)
                     want_row = min(32 * mb + i32, rows_here - 1)
                     assert lds.get(slot) == (want_row, (ks * 16 + kg * 8) * 2), (ks, mb, lane)
     assert len(seen) == sum((c + ROWS - 1) // ROWS for c in counts) * tiles_n
@@ -129,16 +150,39 @@ CASES = [[160] * 8, [136, 108, 150, 121, 132, 111, 130, 136], [1, 0, 255, 257, 3
                                      223, 224, 225, 255, 256]]
 
 
+@pytest.mark.parametrize("waves", [4, 8])
 @pytest.mark.parametrize("case", range(len(CASES)))
-def test_fixed_row_counts(case):
+def test_fixed_row_counts(case, waves):
     for k in (128, 4096, 14336):
-        check(CASES[case], k)
+        check(CASES[case], k, waves=waves)
 
 
 def test_random_row_counts():
     rng = np.random.default_rng(0)
     for _ in range(25):
-        check([int(v) for v in rng.integers(0, 600, size=rng.integers(1, 9))], 4096, tiles_n=2)
+        tiles_n = int(rng.integers(1, 20))
+        check([int(v) for v in rng.integers(0, 600, size=rng.integers(1, 9))], 4096, tiles_n=tiles_n,
+              chunk=[None, tiles_n, 1, 3][int(rng.integers(0, 4))], waves=int(rng.choice([4, 8])))
+
+
+def test_tile_order_keeps_an_xcd_on_few_row_tiles_and_shares_even():
+    """Eight groups of uneven size, 112 column tiles (the fused gate/up launch of a Mixtral layer): every XCD gets 14
+    column tiles of every group, and 32 consecutive workgroups of an XCD touch at most four groups."""
+    counts = [141, 124, 137, 122, 123, 151, 116, 110]
+    offs = [0] + [int(v) for v in np.cumsum(counts)]
+    tiles_n, chunk = 112, 14
+    per_xcd = [[] for _ in range(8)]
+    for b in range(grouped_grid(sum(counts) // ROWS + len(counts), tiles_n, chunk)):
+        t = grouped_tile(offs, tiles_n, chunk, b)
+        if t is not None:
+            per_xcd[b & 7].append(t[0])
+    for seq in per_xcd:
+        assert sorted(seq) == sorted(list(range(8)) * 14)
+        assert max(len(set(seq[i:i + 32])) for i in range(len(seq))) <= 4
+    # a launch of a single round (the down projection: 16 column tiles): a group's column tiles share an XCD
+    for b in range(grouped_grid(12, 16, 16)):
+        t = grouped_tile(offs, 16, 16, b)
+        assert t is None or t[0] == b & 7
 
 
 # ---- dense 128-row form: the line of tiles dealt to the XCDs, whole or in 64-row halves (lowbit_gemm_kernel.h,
