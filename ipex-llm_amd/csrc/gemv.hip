@@ -70,11 +70,59 @@ template <int QT> struct UnpackInt4Bf16 {
 template <> struct Unpack<QT_SYM_INT4, __bf16> : UnpackInt4Bf16<QT_SYM_INT4> {};
 template <> struct Unpack<QT_ASYM_INT4, __bf16> : UnpackInt4Bf16<QT_ASYM_INT4> {};
 
-// nf4: code-book lookup from a 16-entry table in LDS (entries already in the activation type).
+// nf4: code-book lookup, two ways.
+//   - From a 16-entry table in LDS: eight 2-byte reads and about twelve vector instructions per dword of codes.
+//   - In registers: the 16 entries, already in the activation type, lie in two byte planes (low bytes, high bytes)
+//     of four registers each; v_perm_b32 looks four codes up at a time in the eight bytes of a register pair -
+//     entries 0..7 and 8..15 separately, a third v_perm_b32 picks per byte by the code's bit 3 - and two more
+//     interleave the planes into 16-bit values: 21 vector instructions per dword of eight codes, no LDS access.
+// Measured on one MI355X on the Llama-3-70B linear set (419 MB of nf4 weights, bf16): at M = 1 from LDS 115.9 us,
+// in registers 123.0, half of the sub-blocks each way 117.7; at M = 16, where x takes its share of the LDS pipe,
+// 171.4 / 156.7 / 165.6.  So up to four rows of x look up in LDS and more rows in registers.  Either way nf4 stays
+// a quarter behind sym_int4 at the same bytes ([28672 x 8192] at M = 1: 31.7 against 25.5 us): the lookups are
+// instructions the integer formats do not issue, whichever unit takes them.
+struct Nf4Planes {
+    uint32_t lo[4], hi[4];        // byte i % 4 of register i / 4 = low / high byte of entry i
+    uint32_t k04, k0123;          // 0x04040404 and 0x03020100 in vector registers: as literals the two would need the
+                                  // one constant slot of v_and_or_b32 twice
+};
+// RESID: what rounding the code book to AT dropped (the second term of the fp32-output variants)
+template <typename AT, bool RESID> __device__ inline Nf4Planes nf4_planes() {
+    Nf4Planes t = {};
+#pragma unroll
+    for (int i = 0; i < 16; i++) {                      // (constants: folded at compile time)
+        const AT main = to_at<AT>(NF4_CODEBOOK[i]);
+        const AT v = RESID ? to_at<AT>(NF4_CODEBOOK[i] - (float)main) : main;
+        const uint32_t b = __builtin_bit_cast(uint16_t, v);
+        t.lo[i / 4] |= (b & 0xffu) << (8 * (i % 4));
+        t.hi[i / 4] |= (b >> 8) << (8 * (i % 4));
+    }
+    asm("v_mov_b32 %0, 0x04040404" : "=v"(t.k04));
+    asm("v_mov_b32 %0, 0x03020100" : "=v"(t.k0123));
+    return t;
+}
 template <typename AT> struct Unpack<QT_NF4, AT> {
     static constexpr float OFFSET = 0.0f;
-    __device__ static typename Vec8<AT>::type run(uint32_t v, const void *lut_, uint32_t) {
-        const AT *lut = (const AT *)lut_;
+    // four codes, one per byte of `sel` (bits 0..2) and `mrg` (0x03020100 + 4 * bit 3 per byte) -> one byte plane
+    __device__ static uint32_t plane4(const uint32_t (&p)[4], uint32_t sel, uint32_t mrg) {
+        return __builtin_amdgcn_perm(__builtin_amdgcn_perm(p[3], p[2], sel), __builtin_amdgcn_perm(p[1], p[0], sel), mrg);
+    }
+    __device__ static typename Vec8<AT>::type run(uint32_t v, const void *planes_, uint32_t) {
+        const Nf4Planes &t = *(const Nf4Planes *)planes_;
+        // nibbles 0, 2, 4, 6 (columns 0, 4, 1, 5) are the low nibbles of the four bytes, 1, 3, 5, 7 (columns 2, 6,
+        // 3, 7) the high ones
+        const uint32_t sel_e = v & 0x07070707u, mrg_e = and_or(v >> 1, t.k04, t.k0123);
+        const uint32_t sel_o = (v >> 4) & 0x07070707u, mrg_o = and_or(v >> 5, t.k04, t.k0123);
+        const uint32_t lo_e = plane4(t.lo, sel_e, mrg_e), hi_e = plane4(t.hi, sel_e, mrg_e);
+        const uint32_t lo_o = plane4(t.lo, sel_o, mrg_o), hi_o = plane4(t.hi, sel_o, mrg_o);
+        u32x4 r;
+        r[0] = __builtin_amdgcn_perm(hi_e, lo_e, 0x06020400u);      // columns 0, 1: bytes 0 and 2 of the even set
+        r[1] = __builtin_amdgcn_perm(hi_o, lo_o, 0x06020400u);      // columns 2, 3
+        r[2] = __builtin_amdgcn_perm(hi_e, lo_e, 0x07030501u);      // columns 4, 5: bytes 1 and 3
+        r[3] = __builtin_amdgcn_perm(hi_o, lo_o, 0x07030501u);      // columns 6, 7
+        return __builtin_bit_cast(typename Vec8<AT>::type, r);
+    }
+    __device__ static typename Vec8<AT>::type run_lds(uint32_t v, const AT *lut) {
         typename Vec8<AT>::type r;
         r[0] = lut[v & 0xf]; r[2] = lut[(v >> 4) & 0xf]; r[4] = lut[(v >> 8) & 0xf]; r[6] = lut[(v >> 12) & 0xf];
         r[1] = lut[(v >> 16) & 0xf]; r[3] = lut[(v >> 20) & 0xf]; r[5] = lut[(v >> 24) & 0xf]; r[7] = lut[v >> 28];
@@ -190,15 +238,16 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
     // M = 16 a workgroup otherwise pulls 3.5 bytes of x out of L2 per byte of weight)
     constexpr int NW = DUAL ? 2 : R;
     static_assert(!(DUAL && R != 1) && XN * 1024 >= NW * MT * 256, "bad GEMV shape parameters");
-    // nf4 code book in the activation type.  With fp32 output a second table holds what the rounding to AT
-    // dropped, and a second MFMA per sub-block adds it: the weights then carry 16 mantissa bits like x does.
-    __shared__ AT lut[16], lut_lo[16];
-    if constexpr (QT == QT_NF4) {
-        if (threadIdx.x < 16) {
-            const AT hi = to_at<AT>(NF4_CODEBOOK[threadIdx.x]);
-            lut[threadIdx.x] = hi;
-            lut_lo[threadIdx.x] = to_at<AT>(NF4_CODEBOOK[threadIdx.x] - (float)hi);
-        }
+    // nf4 code book in the activation type (byte planes in registers).  With fp32 output a second table holds what
+    // the rounding to AT dropped, and a second MFMA per sub-block adds it: the weights then carry 16 mantissa bits
+    // like x does.
+    const Nf4Planes lut_planes = (QT == QT_NF4) ? nf4_planes<AT, false>() : Nf4Planes{};
+    const Nf4Planes lut_lo_planes = (QT == QT_NF4 && F32OUT) ? nf4_planes<AT, true>() : Nf4Planes{};
+    const void *const lut = &lut_planes, *const lut_lo = &lut_lo_planes;
+    constexpr bool NF4_IN_LDS = QT == QT_NF4 && MT == 1 && !F32OUT;     // (see Unpack<QT_NF4>)
+    __shared__ AT lut_lds[16];
+    if constexpr (NF4_IN_LDS) {
+        if (threadIdx.x < 16) lut_lds[threadIdx.x] = to_at<AT>(NF4_CODEBOOK[threadIdx.x]);
         __syncthreads();
     }
 
@@ -309,7 +358,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     V8 b;
-                    if constexpr (IS4) b = Unpack<QT, AT>::run(tl.q0[j], lut, magic);
+                    if constexpr (NF4_IN_LDS) b = Unpack<QT, AT>::run_lds(tl.q0[j], lut_lds);
+                    else if constexpr (IS4) b = Unpack<QT, AT>::run(tl.q0[j], lut, magic);
                     else if (j < 2) b = Unpack8<QT, AT>::run(tl.q0[2 * j], tl.q0[2 * j + 1]);
                     else b = Unpack8<QT, AT>::run(tl.q1[2 * (j - 2)], tl.q1[2 * (j - 2) + 1]);
                     float d, mn;

@@ -96,10 +96,15 @@ static int launch_grouped_mlp_t(const void *x, const void *const *wg, const void
     const int chunk = grouped_chunk(tiles_n, plan.one_round);
     const GroupArgs ga = {offsets, (const uint8_t *const *)wg, (const uint8_t *const *)wu, n_groups, act, 0, chunk};
     const int n_wg = grouped_grid(grouped_max_row_tiles(total_rows, n_groups, GM_TALL), tiles_n, chunk);
-    if (plan.waves == 8)
+    // nf4 always takes the eight-wave form: its two waves per SIMD cover each other's code book reads (the dense
+    // tall form gains 5-9 % from it), and with four waves, two weight blocks and the lookups' temporaries the fused
+    // kernel sits at the register limit, where the compiler has moved accumulator blocks around inside the loop.
+    if (plan.waves == 8 || QT == QT_NF4) {
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL, true, true, 8>), dim3(n_wg), dim3(512), 0, st, (const AT *)x,
                            (const uint8_t *)nullptr, (AT *)y, 0, N, K, 1, ga, G, (float *)nullptr, 0, tiles_n);
-    else
+        return 0;
+    }
+    if constexpr (QT != QT_NF4)
         hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL, true, true>), dim3(n_wg), dim3(256), 0, st, (const AT *)x,
                            (const uint8_t *)nullptr, (AT *)y, 0, N, K, 1, ga, G, (float *)nullptr, 0, tiles_n);
     return 0;
