@@ -92,6 +92,9 @@ def main():
                     help="run only the batch-sized product (M=32, 64, 128 on [11008 x 4096], sym_int4, fp16)")
     ap.add_argument("--quantize-only", action="store_true",
                     help="run only the block quantizer (fp32 [11008 x 4096] -> sym_int4, tiled) and print its rate")
+    ap.add_argument("--floor-only", action="store_true",
+                    help="run the serialized [11008 x 4096] GEMV loop next to what launches that only READ the same bytes "
+                         "cost in the same chain (libstream_floor.so: an empty kernel, twelve read patterns)")
     ap.add_argument("--moe-only", action="store_true",
                     help="run only the Mixtral expert FFN legs (fp8_e4m3, 512 tokens top-2, and one token)")
     args = ap.parse_args()
@@ -340,6 +343,33 @@ def main():
                 "how": "HIP events around graph replays of 64 chained launches over 64 distinct weights"}
     if args.roofline_only:
         print(json.dumps({"roofline": roofline}))
+        return
+    if args.floor_only:
+        # The same chain - one launch per distinct weight, 64 per graph replay, HIP events around the replays - with
+        # launches that do nothing, and with launches that read the weight's bytes (rounded down to 16) and nothing else.
+        floor = ctypes.CDLL(os.path.join(ROOT, "ipex-llm_amd", "ipex_llm", "libs", "libstream_floor.so"))
+        floor.stream_floor_pattern_name.restype = ctypes.c_char_p
+        floor.stream_floor_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        floor.stream_floor_empty.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        nbytes = hb // 16 * 16
+
+        def chain(launch):
+            def run():
+                st = stream()
+                for b in gu:
+                    assert launch(b, st) == 0
+            return time_graph(capture(run), max(5, args.steps), max(3, args.warmup)) * 1e3 / len(gu)
+        res = {"gemv_us": round(us, 3), "bytes": hb,
+               "empty_launch_us": round(chain(lambda b, st: floor.stream_floor_empty(sink.data_ptr(), st)), 3), "reads_us": {}}
+        for p in range(floor.stream_floor_patterns()):
+            res["reads_us"][floor.stream_floor_pattern_name(p).decode()] = round(
+                chain(lambda b, st: floor.stream_floor_read(b.data_ptr(), nbytes, p, sink.data_ptr(), st)), 3)
+        best = min(res["reads_us"].values())
+        res["fastest_read_us"], res["slowest_read_us"] = best, max(res["reads_us"].values())
+        res["fastest_read_frac_of_hbm_peak"] = round(nbytes / (best * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+        res["gemv_frac_of_hbm_peak"] = roofline["frac"]
+        print(json.dumps({"floor": res}))
         return
 
     ms = time_graph(capture(lambda: sweep(args.m, xs, ys)), args.steps, args.warmup)

@@ -187,6 +187,11 @@ int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout,
 #define LOWBIT_PLAN_RING 1
 #define LOWBIT_PLAN_GEMM 2
 #define LOWBIT_PLAN_GEMM_SPLIT 3
+/* What lowbit_forward_ws makes use of when the caller can spare at most max_bytes of workspace for this format
+ * and shape: the size of the partial tiles of the plan it then picks, 0 when that plan has none.  A caller
+ * with a budget asks this instead of capping lowbit_workspace_bytes (which carries no format and returns the most
+ * any format could use): what it passes on is then exactly what the plan was made for. */
+size_t lowbit_workspace_bytes_for(int qtype, int layout, int64_t M, int64_t N, int64_t K, size_t max_bytes);
 int lowbit_forward_plan(int qtype, int layout, int64_t M, int64_t N, int64_t K, int have_workspace,
                         size_t workspace_bytes);
 /* The two kernels behind lowbit_forward, for callers (and benchmarks) that choose themselves.

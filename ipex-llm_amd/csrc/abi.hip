@@ -282,6 +282,23 @@ static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, 
     return PLAN_GEMM;
 }
 
+// What lowbit_forward_ws will use of a workspace of at most max_bytes for this format and shape: the bytes of the
+// plan it then picks (0 when that plan leaves no partial tiles).
+extern "C" size_t lowbit_workspace_bytes_for(int qtype, int layout, int64_t M, int64_t N, int64_t K, size_t max_bytes) {
+    if (!qk_size(qtype) || M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;
+    int splits = 1;
+    if (max_bytes < 16) return 0;
+    switch (plan_forward(qtype, layout, M, N, K, true, max_bytes, true, &splits)) {
+    case PLAN_RING: {
+        // (a run that cuts no tile needs no bytes, but the plan is only made for a caller that brings a workspace)
+        const size_t need = ring_workspace_bytes((int)M, (int)N, (int)K, 0);
+        return need ? need : 16;
+    }
+    case PLAN_GEMM_SPLIT: return split_bytes(M, N, splits);
+    default: return 0;
+    }
+}
+
 extern "C" int lowbit_forward_plan(int qtype, int layout, int64_t M, int64_t N, int64_t K, int have_workspace,
                                    size_t workspace_bytes) {
     if (!qk_size(qtype) || M < 0 || N < 0 || K < 0) return -1;

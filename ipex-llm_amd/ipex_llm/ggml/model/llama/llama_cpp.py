@@ -210,6 +210,15 @@ _lib.lowbit_forward_plan.restype = c_int
 PLAN_GEMV, PLAN_RING, PLAN_GEMM, PLAN_GEMM_SPLIT = 0, 1, 2, 3
 
 
+_lib.lowbit_workspace_bytes_for.argtypes = [c_int, c_int, c_int64, c_int64, c_int64, c_size_t]
+_lib.lowbit_workspace_bytes_for.restype = c_size_t
+
+
+def lowbit_workspace_bytes_for(qtype, layout, m, n, k, max_bytes) -> int:
+    """Bytes of workspace lowbit_forward_ws uses for this format when it may have at most max_bytes."""
+    return int(_lib.lowbit_workspace_bytes_for(qtype, layout, m, n, k, max_bytes))
+
+
 def lowbit_forward_plan(qtype, layout, m, n, k, have_workspace, workspace_bytes=0) -> int:
     """PLAN_* code of the kernel lowbit_forward (have_workspace False) / lowbit_forward_ws would run."""
     return _lib.lowbit_forward_plan(qtype, layout, m, n, k, int(bool(have_workspace)), workspace_bytes)

@@ -152,18 +152,23 @@ def ggml_q_format_convet_cpu2xpu(tensor: torch.Tensor, num_elem: int, qtype: int
     """ggml layout -> device layout (reference: low_bit_linear.py:178-204).
 
     `shape` = (out_features, in_features) is an addition: the tiled device layout interleaves
-    16 rows, which the reference's (num_elem, qtype) pair cannot describe."""
+    16 rows, which the reference's (num_elem, qtype) pair cannot describe.  Called with the reference's
+    three arguments it does what the C symbol of the same name does: a copy that stays in the ggml
+    layout, which is a valid device weight (layout 0, the any-shape kernels)."""
     _check_blob_dtype(tensor, qtype)
-    invalidInputError(shape is not None and reduce(mul, shape, 1) == num_elem,
-                      "the MI355X device layout depends on the weight shape: pass shape=(out, in)")
+    if shape is None:
+        return tensor.clone()
+    invalidInputError(reduce(mul, shape, 1) == num_elem, "shape does not hold num_elem weights")
     return _relayout(tensor, qtype, shape, ggml.LAYOUT_GGML)
 
 
 def ggml_q_format_convet_xpu2cpu(tensor: torch.Tensor, num_elem: int, qtype: int, shape=None):
-    """device layout -> ggml layout (reference: low_bit_linear.py:207-233)."""
+    """device layout -> ggml layout (reference: low_bit_linear.py:207-233).  Without `shape` the blob
+    is taken to be in the ggml layout already (what the three-argument cpu2xpu call leaves): a copy."""
     _check_blob_dtype(tensor, qtype)
-    invalidInputError(shape is not None and reduce(mul, shape, 1) == num_elem,
-                      "the MI355X device layout depends on the weight shape: pass shape=(out, in)")
+    if shape is None:
+        return tensor.clone()
+    invalidInputError(reduce(mul, shape, 1) == num_elem, "shape does not hold num_elem weights")
     return _relayout(tensor, qtype, shape, ggml.LAYOUT_TILED)
 
 
@@ -250,8 +255,8 @@ def forward_new(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int, 
         with torch.cuda.device(x.device):
             # workspace for the fp32 partial tiles of the batch-size kernel and of the GEMM when it
             # splits K; taken from torch's caching allocator, so steady-state calls do not allocate
-            ws_bytes = ggml.lowbit_workspace_bytes(m, output_size, k) if layout == ggml.LAYOUT_TILED else 0
-            ws_bytes = min(ws_bytes, _WORKSPACE_CAP)
+            # (the library is told the budget and says what the plan it makes within it needs)
+            ws_bytes = ggml.lowbit_workspace_bytes_for(qtype, layout, m, output_size, k, _WORKSPACE_CAP)
             if ws_bytes:
                 ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
                 ggml.lowbit_forward_ws(xc.data_ptr(), w.data_ptr(), y.data_ptr(), qtype, layout, _DT[xc.dtype],
@@ -509,6 +514,27 @@ class MatMulLowBit(torch.autograd.Function):
         return grad_A, None, None
 
 
+class MatMulLowBitCPU(torch.autograd.Function):
+    """The same for a weight blob that lives on the host (reference: low_bit_linear.py:544-570): forward through
+    the ggml-style host-pointer matmul, backward = grad_out times the dequantized weight."""
+
+    @staticmethod
+    def forward(ctx, A, weight):
+        ctx.tensors = (A, weight) if any(ctx.needs_input_grad[:2]) else (None, None)
+        x_2d = A.detach().reshape(-1, A.shape[-1])
+        result = ggml_matmul_src1_x_src0_t(weight.data, x_2d.cpu(), weight._shape, weight.qtype)
+        return result.view(A.shape[:-1] + (weight._shape[0],)).to(A.device)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        A, weight = ctx.tensors
+        grad_A = None
+        if ctx.needs_input_grad[0]:
+            dequant_weight = ggml_convert_fp32(weight.data, weight._shape, weight._shape[0] * weight._shape[1], weight.qtype)
+            grad_A = torch.matmul(grad_output, dequant_weight.to(grad_output.dtype).to(grad_output.device))
+        return grad_A, None
+
+
 class LowBitLinear(nn.Linear):
     """nn.Linear whose weight is a packed low-bit blob (reference: low_bit_linear.py:573-715)."""
 
@@ -590,8 +616,17 @@ class LowBitLinear(nn.Linear):
             invalidInputError(self.qtype not in (NF3, NF4, FP8E4, FP4, FP8E5),
                               "NF3, NF4, FP4 and FP8 quantization are currently not supported on CPU")
             invalidInputError(self.weight.quantized, "the weight has not been quantized yet: call .to() first")
-            result = ggml_matmul_src1_x_src0_t(self.weight.data, x_2d.cpu(), self.weight_shape, self.qtype)
-            result = result.view(new_shape).to(x.device)
+            if is_training and x.requires_grad:
+                result = MatMulLowBitCPU.apply(x, self.weight)
+            elif self.qtype == SYM_INT4 and x_2d.shape[0] >= TORCH_LINEAR_THRESHOLD:
+                # many rows against a host-resident weight: dequantize once and let the dense fp32 product
+                # run where x is (reference: low_bit_linear.py:699-702) - every 16 rows would otherwise cost a
+                # pass over the weight behind a copy of x and y across PCIe
+                x0_fp32 = ggml_int4_convert_fp32(self.weight.data, self.weight_shape, self.weight_length)
+                result = F.linear(x.to(dtype=x0_fp32.dtype), x0_fp32.to(x.device))
+            else:
+                result = ggml_matmul_src1_x_src0_t(self.weight.data, x_2d.cpu(), self.weight_shape, self.qtype)
+                result = result.view(new_shape).to(x.device)
             invalidInputError(self.mp_group is None,
                               "mp_group (tensor parallel all-reduce) is outside this single-GPU build")
             if self.bias is not None:

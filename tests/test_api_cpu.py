@@ -433,3 +433,32 @@ def test_grouped_split_workspace_holds_a_tile_for_every_workgroup():
                 assert tall == 1 and splits * grid * tile <= ws, (n_groups, rows, n, k, ws, splits, grid)
         assert (need == 0) == (ggml.lowbit_grouped_forward_plan(n_groups, rows, n, k, True, 1 << 40)[1] == 1)
     assert split_seen
+
+
+def test_layout_converters_take_the_reference_signature():
+    """ggml_q_format_convet_cpu2xpu(tensor, num_elem, qtype) as the reference calls it (low_bit_linear.py:178-233)
+    does what the C symbol of that name does: a copy that stays in the ggml layout."""
+    from ipex_llm.transformers.low_bit_linear import ggml_q_format_convet_cpu2xpu, ggml_q_format_convet_xpu2cpu
+    blob = torch.arange(18 * 8, dtype=torch.uint8)
+    for fn in (ggml_q_format_convet_cpu2xpu, ggml_q_format_convet_xpu2cpu):
+        out = fn(blob, 256, Q["sym_int4"])
+        assert torch.equal(out, blob) and out.data_ptr() != blob.data_ptr()
+    with pytest.raises(RuntimeError, match="uint8"):
+        ggml_q_format_convet_cpu2xpu(blob.float(), 256, Q["sym_int4"])
+
+
+def test_workspace_query_with_a_budget_names_what_the_plan_uses():
+    """lowbit_workspace_bytes_for(qtype, layout, M, N, K, budget): never above the budget, zero where the plan has
+    no partial tiles, and the plan made with exactly that many bytes is the plan made with the whole budget."""
+    G, R, D, S = ggml.PLAN_GEMV, ggml.PLAN_RING, ggml.PLAN_GEMM, ggml.PLAN_GEMM_SPLIT
+    for qtype in (2, 3, 8, 10, 15):
+        for n, k in ((4096, 4096), (11008, 4096), (4096, 11008), (1024, 8192), (28672, 8192)):
+            for m in (1, 16, 24, 64, 128, 512, 2048):
+                for budget in (0, 1 << 20, 64 << 20, 256 << 20, 1 << 40):
+                    need = ggml.lowbit_workspace_bytes_for(qtype, 1, m, n, k, budget)
+                    assert need <= budget
+                    plan = ggml.lowbit_forward_plan(qtype, 1, m, n, k, budget >= 16, budget)
+                    assert (need > 0) == (plan in (R, S)), (qtype, m, n, k, budget, need, plan)
+                    assert ggml.lowbit_forward_plan(qtype, 1, m, n, k, need > 0, need) == (plan if need else ggml.lowbit_forward_plan(qtype, 1, m, n, k, False))
+                assert ggml.lowbit_workspace_bytes_for(qtype, 1, m, n, k, 1 << 40) <= ggml.lowbit_workspace_bytes(m, n, k)
+        assert ggml.lowbit_workspace_bytes_for(qtype, 0, 512, 4096, 4096, 1 << 30) == 0      # ggml layout: any-shape kernel

@@ -200,6 +200,34 @@ def test_from_pretrained_tiny_llama_and_low_bit_round_trip(tmp_path):
     assert torch.equal(got, got2)
 
 
+def test_host_resident_weight_takes_the_reference_cpu_routes():
+    """A LowBitLinear whose blob stays on the host (reference: low_bit_linear.py:683-715): few rows go through the
+    ggml-style host-pointer matmul, BIGDL_LLM_LINEAR_THRESHOLD rows and more of sym_int4 through one dequantization
+    and a dense fp32 product, a training step through MatMulLowBitCPU; all three equal the dense layer of the
+    oracle's dequantized weight."""
+    from ipex_llm.transformers import low_bit_linear as lbl
+    n, k = 96, 256
+    w = weights(7300, (n, k))
+    layer = _layer(w, Q["sym_int4"])
+    layer.weight = layer.weight.to("cpu")                     # quantized, still on the host
+    assert layer.weight.data.device.type == "cpu" and layer.weight.quantized
+    wd = torch.from_numpy(orc.dequantize(orc.quantize(w, Q["sym_int4"]), Q["sym_int4"], (n, k)))
+    x_small = torch.randn(5, k)
+    x_large = torch.randn(lbl.TORCH_LINEAR_THRESHOLD, k)
+    for x in (x_small, x_large):
+        y = layer(x)
+        want = x @ wd.t()
+        assert y.shape == want.shape and y.dtype == x.dtype
+        assert (y - want).abs().max() <= 1e-2 * want.abs().max()
+    assert torch.allclose(layer(x_large), x_large @ wd.t(), atol=1e-4)          # the dense route is exact fp32
+    layer.train()
+    xg = torch.randn(3, k, requires_grad=True)
+    y = layer(xg)
+    go = torch.randn_like(y)
+    y.backward(go)
+    assert torch.allclose(xg.grad, go @ wd, atol=1e-4)
+
+
 def test_tiny_llama_generates_under_inference_mode(tmp_path):
     """Callers of the reference run `generate` inside `torch.inference_mode()`: activations are inference
     tensors there (no version counter) and nothing of a layer's merged q/k/v product may outlive the layer."""
