@@ -228,6 +228,20 @@ def main():
         leg["hbm_floor"] = hbm(wb, ms)
         leg["rows_per_expert"] = [int(v) for v in (offsets[1:] - offsets[:-1]).tolist()]
         leg["three_separate_launches_ms"] = round(time_graph(capture(moe_unfused), 10, 2), 4)
+        # what launches that only READ the gate and up weights, in the pattern the grouped GEMM walks them, take
+        # (libstream_floor.so; the fused gate/up launch reads the same bytes and multiplies)
+        floor_path = os.path.join(ROOT, "ipex-llm_amd", "ipex_llm", "libs", "libstream_floor.so")
+        if os.path.exists(floor_path):
+            floor = ctypes.CDLL(floor_path)
+            floor.stream_floor_read_tiles.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                      ctypes.c_void_p, ctypes.c_void_p]
+            sink = torch.zeros(4, dtype=torch.int32, device=dev)
+            both = torch.cat([ptrs["w1"], ptrs["w3"]])
+
+            def read_gate_up():
+                assert floor.stream_floor_read_tiles(both.data_ptr(), 2 * n_exp, ffn // 16, hid // 128, 2112,
+                                                     sink.data_ptr(), stream()) == 0
+            leg["gate_up_weights_read_only_ms"] = round(time_graph(capture(read_gate_up), 10, 2), 4)
         res["mixtral_moe_fp8_512tok_top2"] = leg
         # the same experts at decode: one token through its top-2 experts in two launches (xe_linear.moe_forward_vec);
         # 16 different expert pairs per graph replay, so that the weights come from HBM

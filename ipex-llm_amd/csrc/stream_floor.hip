@@ -31,6 +31,27 @@ __global__ __launch_bounds__(64 * WAVES) void floor_read_kernel(const u32x4 *__r
     if (a == 0x12345678u) out[0] = a;              // (keeps the loads alive; the buffers never hold this value)
 }
 
+// The weight access pattern of the grouped GEMM (lowbit_gemm_kernel.h): a workgroup of four waves owns 16 tile rows
+// (256 weight rows), a wave walks its four tile rows side by side, one tile of each per K step (the first two KiB
+// of a tile: the codes of an 8-bit format).  tiles_per_row tiles of tile_bytes bytes per tile row.
+__global__ __launch_bounds__(256) void floor_read_tiles_kernel(const uint8_t *const *__restrict__ weights, uint32_t *out,
+                                                               int tile_rows, int tiles_per_row, int tile_bytes) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint8_t *w = weights[blockIdx.y];                   // one weight per blockIdx.y, as one expert's
+    const int64_t r0 = ((int64_t)blockIdx.x * 4 + wave) * 4;
+    if (r0 + 4 > tile_rows) return;
+    u32x4 acc = {0, 0, 0, 0};
+#pragma unroll 2
+    for (int s = 0; s < tiles_per_row; s++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const uint8_t *t = w + ((r0 + r) * tiles_per_row + s) * (int64_t)tile_bytes;
+            acc ^= *(const u32x4 *)(t + lane * 16);
+            acc ^= *(const u32x4 *)(t + 1024 + lane * 16);
+        }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) out[0] = 1;
+}
+
 __global__ void floor_empty_kernel(uint32_t *out) {
     if (out == nullptr) __builtin_trap();          // never: a kernel with no work at all
 }
@@ -74,6 +95,18 @@ int stream_floor_read(const void *buf, size_t bytes, int p, void *out, void *str
     case 11: return launch_read<16, 8, 0>(buf, bytes, o, st);
     default: return -1;
     }
+}
+
+// One launch that reads n_weights tiled weights (a table of device pointers in device memory; each tile_rows rows
+// of tiles_per_row tiles, tile_bytes >= 2048 each, tile_rows a multiple of 16) the way the grouped GEMM walks them.
+int stream_floor_read_tiles(const void *const *weights, int n_weights, int tile_rows, int tiles_per_row, int tile_bytes,
+                            void *out, void *stream) {
+    if (!weights || !out || n_weights <= 0 || n_weights > 65535 || tile_rows <= 0 || (tile_rows % 16) || tiles_per_row <= 0 ||
+        tile_bytes < 2048 || (tile_bytes % 16))
+        return -1;
+    hipLaunchKernelGGL(floor_read_tiles_kernel, dim3(tile_rows / 16, n_weights), dim3(256), 0, (hipStream_t)stream,
+                       (const uint8_t *const *)weights, (uint32_t *)out, tile_rows, tiles_per_row, tile_bytes);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 int stream_floor_empty(void *out, void *stream) {
