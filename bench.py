@@ -580,6 +580,29 @@ def cpu_baseline(mods, m, ggml, torch):
             if dt > budget_s:
                 return passes, dt
 
+    def l3_note(working_set_bytes):
+        """Whether a repeated pass over `working_set_bytes` stays in the host's last-level caches (then the rate is
+        a cache rate, not a DRAM rate): the sum of the distinct L3 instances the visible cores report."""
+        total = 0
+        try:
+            seen = set()
+            for cpu in sorted(os.listdir("/sys/devices/system/cpu")):
+                base = f"/sys/devices/system/cpu/{cpu}/cache/index3"
+                if not os.path.isdir(base):
+                    continue
+                shared = open(base + "/shared_cpu_list").read().strip()
+                if shared in seen:
+                    continue
+                seen.add(shared)
+                size = open(base + "/size").read().strip()
+                total += int(size[:-1]) * (1 << 10 if size.endswith("K") else 1 << 20 if size.endswith("M") else 1)
+        except Exception:  # noqa: BLE001
+            total = 0
+        if not total:
+            return f"working set {working_set_bytes >> 20} MiB, host L3 size unknown"
+        fits = "fits" if working_set_bytes <= total else "does not fit"
+        return f"working set {working_set_bytes >> 20} MiB {fits} the host's {total >> 20} MiB of L3 (repeated passes)"
+
     blobs = [(n, k, host_blob(n, k, blob, SYM_INT4)) for name, n, k, blob in mods]
     xs = {k: rng.standard_normal((m, k)).astype(np.float32) for k in (4096, 11008)}
     nbytes = sum(b.size + m * k * 2 + m * n * 2 for n, k, b in blobs)
@@ -591,13 +614,14 @@ def cpu_baseline(mods, m, ggml, torch):
     out = {"value": round(nbytes * passes / dt / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
            "cpu": model, "isa": isa,
            "sample": f"1 of 32 layers (7 linears, {nbytes} algorithmic bytes) x {passes} passes, "
-                     f"oracle ggml-style Q8_0-activation matmul, OpenMP"}
+                     f"oracle ggml-style Q8_0-activation matmul, OpenMP; {l3_note(sum(b.size for _, _, b in blobs))}"}
     more = {}
     # configs[0]: [4096 x 4096], M = 1
     n, k, b = blobs[0]
     x1 = rng.standard_normal((1, k)).astype(np.float32)
     p, t = timed(lambda: orc.mul_mat_q(b, x1, (n, k), SYM_INT4), 2.0)
-    more["single_N4096_K4096_M1"] = {"GB/s": round((b.size + 2 * (n + k)) * p / t / 1e9, 2), "sample": f"{p} calls"}
+    more["single_N4096_K4096_M1"] = {"GB/s": round((b.size + 2 * (n + k)) * p / t / 1e9, 2),
+                                     "sample": f"{p} calls; {l3_note(b.size)}"}
     # configs[1] at M = 4 / 8: the same layer
     for mm in (4, 8):
         xm = {kk: rng.standard_normal((mm, kk)).astype(np.float32) for kk in (4096, 11008)}
@@ -617,7 +641,8 @@ def cpu_baseline(mods, m, ggml, torch):
     b8 = orc.quantize(w8, QT["sym_int8"])
     x8 = rng.standard_normal((1, 8192)).astype(np.float32)
     p, t = timed(lambda: orc.mul_mat_q(b8, x8, (8192, 8192), QT["sym_int8"]), 2.0)
-    more["llama3_70b_q_proj_sym_int8_M1"] = {"GB/s": round((b8.size + 4 * 8192) * p / t / 1e9, 2), "sample": f"{p} calls"}
+    more["llama3_70b_q_proj_sym_int8_M1"] = {"GB/s": round((b8.size + 4 * 8192) * p / t / 1e9, 2),
+                                             "sample": f"{p} calls; {l3_note(b8.size)}"}
     # the block quantizer (ggml_quantize_tensor): GB/s of fp32 input + blob output
     p, t = timed(lambda: orc.quantize(w8, SYM_INT4), 2.0)
     more["quantize_sym_int4_8192x8192"] = {"GB/s": round((w8.nbytes + blob_bytes(8192, 8192)) * p / t / 1e9, 2),
