@@ -112,51 +112,10 @@ size_t ggml_quantize_tensor_rtn_with_weights(const float *src, void *dst, float 
                                              int64_t *hist, bool scale_search, const float *weights);
 /* llama_cpp.py:1081 resolves this name (a restype assignment, no prototype, no caller).  Placeholder that aborts. */
 void ggml_quantize_q4_0(void);
-/* llama.cpp's model API, resolved by llama_cpp.py:228-940 at import and outside the low-bit linear path.
- * Exported so that the import succeeds with LLAMA_CPP_LIB pointing here; the real prototypes differ - these
- * are placeholders that print the name and abort when called. */
-void llama_apply_lora_from_file(void);
-void llama_context_default_params(void);
-void llama_copy_state_data(void);
-void llama_eval(void);
-void llama_free(void);
-void llama_get_embeddings(void);
-void llama_get_kv_cache_token_count(void);
-void llama_get_logits(void);
-void llama_get_state_size(void);
-void llama_init_candidates(void);
-void llama_init_from_file(void);
-void llama_load_session_file(void);
-void llama_mlock_supported(void);
-void llama_mmap_supported(void);
-void llama_model_quantize(void);
-void llama_n_ctx(void);
-void llama_n_embd(void);
-void llama_n_vocab(void);
-void llama_print_system_info(void);
-void llama_print_timings(void);
-void llama_reset_timings(void);
-void llama_sample_frequency_and_presence_penalties(void);
-void llama_sample_repetition_penalty(void);
-void llama_sample_softmax(void);
-void llama_sample_tail_free(void);
-void llama_sample_temperature(void);
-void llama_sample_token(void);
-void llama_sample_token_greedy(void);
-void llama_sample_token_mirostat(void);
-void llama_sample_token_mirostat_v2(void);
-void llama_sample_top_k(void);
-void llama_sample_top_p(void);
-void llama_sample_typical(void);
-void llama_save_session_file(void);
-void llama_set_rng_seed(void);
-void llama_set_state_data(void);
-void llama_time_us(void);
-void llama_token_bos(void);
-void llama_token_eos(void);
-void llama_token_nl(void);
-void llama_token_to_str(void);
-void llama_tokenize(void);
+/* The library also exports the 45 names of llama.cpp's model API that llama_cpp.py:228-940 resolves at import
+ * (llama_eval, llama_tokenize, ...), so that the import succeeds with LLAMA_CPP_LIB pointing here.  They are outside
+ * the low-bit linear path and are not part of this interface: no prototypes are given, and each prints its name
+ * and aborts when called (abi.hip). */
 
 /* ------------------------------------------------------------------ (2) */
 
