@@ -71,10 +71,13 @@ def vregs(spec):
 
 
 def mfma_loops(lines):
-    """Line numbers that lie inside a loop holding an MFMA, from the loop comments the compiler puts behind block
-    labels ('=>This Inner Loop Header', 'in Loop: Header=BB1_23', also on the '; %bb.N:' lines of blocks that
-    are fallen into)."""
+    """Line numbers that lie inside an innermost loop holding an MFMA (a walk along K), from the loop comments the
+    compiler puts behind block labels ('=>This Inner Loop Header', 'in Loop: Header=BB1_23', also on the '; %bb.N:'
+    lines of blocks that are fallen into; a nested loop's header carries 'Parent Loop BB1_5' and its own
+    'Loop Header' on the comment line below).  A loop around such loops - a workgroup that takes one tile after the
+    other - is not one: what it holds besides them runs once per tile."""
     loop_of = {}                                   # line -> header name of the innermost loop it is in
+    parents = set()
     current = None
     for no, line in enumerate(lines):
         t = line.strip()
@@ -82,15 +85,23 @@ def mfma_loops(lines):
         if m:
             rest = m.group(2)
             h = re.search(r"Header=(BB\w+)", rest)
-            if "Loop Header" in rest and m.group(1):
+            par = re.search(r"Parent Loop (BB\w+)", rest)
+            if par:
+                parents.add(par.group(1))
+            below = lines[no + 1].strip() if no + 1 < len(lines) else ""
+            if m.group(1) and ("Loop Header" in rest or (par and below.startswith(";") and "Loop Header" in below)):
                 current = m.group(1)
             elif h:
                 current = h.group(1)
             else:
                 current = None
+        elif t.startswith(";") and "Parent Loop" in t:
+            par = re.search(r"Parent Loop (BB\w+)", t)
+            if par:
+                parents.add(par.group(1))
         if current:
             loop_of[no] = current
-    with_mfma = {h for no, h in loop_of.items() if "v_mfma" in lines[no]}
+    with_mfma = {h for no, h in loop_of.items() if "v_mfma" in lines[no]} - parents
     return {no for no, h in loop_of.items() if h in with_mfma}
 
 

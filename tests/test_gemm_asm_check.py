@@ -108,6 +108,34 @@ def test_the_checker_keeps_checking_after_a_spill_and_tells_loops_from_straight_
     assert "scratch access:" in out.stdout and "inside an MFMA loop" in out.stdout      # nothing allowed: both kinds
 
 
+def test_the_checker_takes_the_innermost_loops_for_the_walks_along_k(tmp_path):
+    """A loop around the K loops (a workgroup that takes tile after tile) holds code that runs once per tile: a
+    spill there is like one outside loops.  The nested loop's header line carries 'Parent Loop', its own 'Loop
+    Header' stands on the comment line below; a reload in it is still an error."""
+    text = ("_Z16gemm_mfma_kernelILi8ELb1ELb0ELi8EEv:\n"
+            ".LBB0_1:                                ; =>This Loop Header: Depth=1\n"
+            "\tscratch_load_dword v2, off, off\n"                   # per tile: allowed when asked for
+            "\tv_mfma_f32_32x32x16_f16 a[16:31], v[0:3], v[4:7], a[16:31]\n"   # (an MFMA outside the K loop)
+            ".LBB0_2:                                ;   Parent Loop BB0_1 Depth=1\n"
+            "                                        ; =>  This Inner Loop Header: Depth=2\n"
+            "%s"
+            "\tv_mfma_f32_32x32x16_f16 a[0:15], v[0:3], v[4:7], a[0:15]\n"
+            "\ts_cbranch_scc1 .LBB0_2\n"
+            "; %%bb.3:                                ;   in Loop: Header=BB0_1 Depth=1\n"
+            "\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n"
+            "\tscratch_store_dword off, v2, off\n"
+            "\ts_cbranch_scc1 .LBB0_1\n"
+            "; %%bb.4:\n"
+            "\ts_endpgm\n")
+    for inner, rc in (("", 0), ("\tscratch_load_dword v1, off, off\n", 1)):
+        f = tmp_path / ("nested%d.s" % rc)
+        f.write_text(text % inner)
+        out = subprocess.run([sys.executable, CHECKER, str(f), "--allow-scratch-outside-loops", "Li8ELb1ELb0ELi8E"],
+                             capture_output=True, text=True)
+        assert out.returncode == rc, out.stdout
+        assert out.stdout.count("inside an MFMA loop") == rc
+
+
 def test_the_checker_counts_the_loads_behind_the_last_lds_dma_of_a_deep_step(tmp_path):
     body = ("_Z16gemm_mfma_kernelv:\n"
             "\tglobal_load_lds_dwordx4 v1, s[0:1]\n"

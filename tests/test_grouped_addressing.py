@@ -48,6 +48,55 @@ def grouped_tile(offs, tiles_n, chunk, b):
     return None
 
 
+def grouped_tile_lanes(offs, tiles_n, chunk, b):
+    """The same answer found the way a wave finds it for up to 64 groups (grouped_tile_lanes): lane e holds group
+    e's offsets, an inclusive prefix sum over the lanes counts whole row tiles, a ballot marks the groups with a
+    partly filled one, and the group comes out of a ballot over 'my range of row tiles holds idx'."""
+    n = len(offs) - 1
+    assert n <= 64
+    lanes = range(64)
+    r0 = [offs[l] if l < n else 0 for l in lanes]
+    r1 = [offs[l + 1] if l < n else 0 for l in lanes]
+    rows = [max(r1[l] - r0[l], 0) for l in lanes]
+    f = [rows[l] // ROWS for l in lanes]
+    p = [rows[l] % ROWS != 0 for l in lanes]
+    incl = list(f)
+    d = 1
+    while d < 64:                                   # shuffle-up scan: lane l adds what lane l - d held before the step
+        prev = list(incl)
+        for l in lanes:
+            if l >= d:
+                incl[l] = prev[l] + prev[l - d]
+        d <<= 1
+    full = incl[63]
+    pm = sum(1 << l for l in lanes if p[l])
+    per_row_tile = (tiles_n + chunk - 1) // chunk
+    cells = (full + bin(pm).count("1")) * per_row_tile
+    i, ci = b >> 3, b & 7
+    while True:
+        if ci >= cells:
+            return None
+        q = ci % per_row_tile
+        size = min(chunk, tiles_n - q * chunk)
+        if i < size:
+            break
+        i -= size
+        ci += 8
+    tn = q * chunk + i
+    idx = ci // per_row_tile
+    want_full = idx < full
+    if want_full:
+        hit = [l for l in lanes if incl[l] - f[l] <= idx < incl[l]]
+    else:
+        idx -= full
+        hit = [l for l in lanes if p[l] and bin(pm & ((1 << l) - 1)).count("1") == idx]
+    if not hit:
+        return None
+    g = hit[0]
+    m0 = r0[g] + ((idx - (incl[g] - f[g])) if want_full else f[g]) * ROWS
+    return g, m0, r1[g], tn
+
+
 def grouped_grid(row_tiles, tiles_n, chunk):
     cells = row_tiles * ((tiles_n + chunk - 1) // chunk)
     return 8 * ((cells + 7) // 8) * chunk
@@ -242,3 +291,22 @@ def test_dense_tile_line_with_half_tiles_covers_every_row_once():
         for split_tail in (0, T // 8 + 1, 3):          # none, all (what the launcher passes), a few at each share's end
             hits = _dense_rows_covered(M, tiles_n, split_tail)
             assert (hits == 1).all(), (M, tiles_n, split_tail)
+
+
+@pytest.mark.parametrize("n_groups", [1, 8, 63, 64])
+def test_lane_lookup_agrees_with_the_walk_over_the_offsets(n_groups):
+    rng = np.random.default_rng(n_groups)
+    for trial in range(6):
+        counts = rng.integers(0, 3 * ROWS, n_groups)
+        counts[rng.random(n_groups) < 0.3] = 0
+        if trial == 0:
+            counts[:] = ROWS                        # whole tiles only
+        if trial == 1:
+            counts[:] = 0                           # nothing at all
+        offs = [0] + [int(v) for v in np.cumsum(counts)]
+        for tiles_n, chunk in ((3, 1), (16, 2), (5, 5)):
+            row_tiles = sum(int(c) // ROWS + (int(c) % ROWS != 0) for c in counts)
+            n_wg = grouped_grid(offs[-1] // ROWS + n_groups, tiles_n, chunk)
+            got = [grouped_tile_lanes(offs, tiles_n, chunk, b) for b in range(n_wg)]
+            assert got == [grouped_tile(offs, tiles_n, chunk, b) for b in range(n_wg)]
+            assert sum(g is not None for g in got) == row_tiles * tiles_n

@@ -123,6 +123,44 @@ def test_grouped_mlp_forward_matches_oracle_per_group(qname, dtype, act, counts)
         r0 += c
 
 
+def _many_counts(n_groups, mean_rows, seed):
+    """Row counts for many groups: a quarter empty, single rows, counts either side of a whole tile, a long tail."""
+    rng = np.random.default_rng(seed)
+    counts = rng.poisson(mean_rows, n_groups)
+    counts[rng.random(n_groups) < 0.25] = 0
+    counts[0], counts[-1] = 1, 2 * mean_rows + 1           # first and last group take part
+    counts[n_groups // 2] = 257
+    return [int(c) for c in counts]
+
+
+@pytest.mark.parametrize("n_groups", [64, 65, 100])
+@pytest.mark.parametrize("mean_rows", [24, 140])
+def test_grouped_launches_find_their_tiles_among_many_groups(n_groups, mean_rows):
+    """Up to 64 groups a workgroup finds its row tile with one lane per group, beyond that by walking the offsets;
+    both forms of tile (up to 96 rows per group on average: 128-row tiles, above: 256-row tiles), plain and fused."""
+    qtype, dtype = Q["sym_int4"], torch.float16
+    n, k = 272, 256
+    counts = _many_counts(n_groups, mean_rows, 100 * n_groups + mean_rows)
+    gate, raw_g = _experts(n_groups, n, k, qtype, 9100)
+    up, raw_u = _experts(n_groups, n, k, qtype, 9300)
+    rows = sum(counts)
+    torch.manual_seed(6)
+    x = torch.randn(rows, k).to(dtype).cuda()
+    offs = _offsets(counts)
+    y = grouped_forward(x, offs, ExpertWeights(gate)).float().cpu().numpy()
+    h = grouped_mlp_forward(x, offs, ExpertWeights(gate), ExpertWeights(up), 0).float().cpu().numpy()
+    r0 = 0
+    for e, c in enumerate(counts):
+        if c:
+            xe = x[r0:r0 + c].float().cpu().numpy()
+            g = orc.mul_mat_exact(orc.quantize(raw_g[e], qtype), xe, (n, k), qtype)
+            u = orc.mul_mat_exact(orc.quantize(raw_u[e], qtype), xe, (n, k), qtype)
+            assert np.abs(y[r0:r0 + c] - g).max() <= 2e-3 * np.abs(g).max(), (e, c)
+            want = g / (1.0 + np.exp(-g)) * u
+            assert np.abs(h[r0:r0 + c] - want).max() <= 2e-3 * np.abs(want).max(), (e, c)
+        r0 += c
+
+
 def test_grouped_ffn_replays_correctly_from_a_hip_graph():
     """The fused gate/up launch and the down projection with its K-split workspace, captured once and replayed
     with new activations and a new routing (static buffers), with eager work and synchronizations between the
