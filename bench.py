@@ -306,7 +306,21 @@ def main():
                 ggml.lowbit_forward(xp.data_ptr(), b.data_ptr(), yp.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED,
                                     ggml.DT_F16, m, 11008, 4096, st)
         ms4 = time_graph(capture(prefill), 10, 10) / len(gu8)     # clocks settle after some tens of launches
-        return mfma(2.0 * m * 11008 * 4096, ms4, kernel="gemm_mfma_kernel<sym_int4,f16> on [11008 x 4096], M=%d" % m)
+        leg = mfma(2.0 * m * 11008 * 4096, ms4, kernel="gemm_mfma_kernel<sym_int4,f16> on [11008 x 4096], M=%d" % m)
+        if m == 2048:
+            # The same kernel on the first 8192 rows of the same weights (the tiled layout keeps 16 rows of the
+            # weight together): 512 tiles of 128 x 256 on the 512 workgroup slots, where [11008 x 4096] has 688.
+            # Its time per tile, times 688 / 512, is what dealing the tiles out evenly could reach at best.
+            def filled():
+                st = stream()
+                for b in gu8:
+                    ggml.lowbit_forward(xp.data_ptr(), b.data_ptr(), yp.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED,
+                                        ggml.DT_F16, m, 8192, 4096, st)
+            ms_f = time_graph(capture(filled), 10, 10) / len(gu8)
+            leg["filled_launch_N8192"] = {"ms": round(ms_f, 4), "frac": round(2.0 * m * 8192 * 4096 / (ms_f * 1e-3) / 2.5e15, 4),
+                                          "tiles": "512 on 512 slots",
+                                          "even_deal_bound_ms": round(ms_f * 688 / 512, 4)}
+        return leg
 
     if args.prefill_only:
         print(json.dumps({"prefill": prefill_leg()}))
