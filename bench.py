@@ -309,8 +309,8 @@ def main():
         leg = mfma(2.0 * m * 11008 * 4096, ms4, kernel="gemm_mfma_kernel<sym_int4,f16> on [11008 x 4096], M=%d" % m)
         if m == 2048:
             # The same kernel on the first 8192 rows of the same weights (the tiled layout keeps 16 rows of the
-            # weight together): 512 tiles of 128 x 256 on the 512 workgroup slots, where [11008 x 4096] has 688.
-            # Its time per tile, times 688 / 512, is what dealing the tiles out evenly could reach at best.
+            # weight together): 256 tiles of 256 x 256, one per CU, where [11008 x 4096] has 344 tiles' worth of work.
+            # Its time, times 344 / 256, is what dealing the tiles out evenly could reach at best.
             def filled():
                 st = stream()
                 for b in gu8:
@@ -318,8 +318,8 @@ def main():
                                         ggml.DT_F16, m, 8192, 4096, st)
             ms_f = time_graph(capture(filled), 10, 10) / len(gu8)
             leg["filled_launch_N8192"] = {"ms": round(ms_f, 4), "frac": round(2.0 * m * 8192 * 4096 / (ms_f * 1e-3) / 2.5e15, 4),
-                                          "tiles": "512 on 512 slots",
-                                          "even_deal_bound_ms": round(ms_f * 688 / 512, 4)}
+                                          "tiles": "256 of 256 x 256 on 256 CUs",
+                                          "even_deal_bound_ms": round(ms_f * 344 / 256, 4)}
         return leg
 
     if args.prefill_only:
