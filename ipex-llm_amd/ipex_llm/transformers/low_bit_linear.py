@@ -204,15 +204,23 @@ def reshape_lm_head_input(x):
 
 
 def use_batch_forward(x: torch.Tensor, qtype: int, output_len: int):
-    """Whether the small-batch kernel serves this call (reference: low_bit_linear.py:272-307).
+    """Whether LowBitLinear.forward hands this call to batch_forward (reference: low_bit_linear.py:272-307).
 
-    On MI355X the streaming kernel takes up to 16 rows of x per pass over the weights and
-    needs no per-device table; the shape rules of the reference are kept."""
+    The reference's window for a device that none of its per-device clauses names (they list Intel GPUs: arc,
+    pvc, mtl, arl, lnl, bmg): float32 or half x with K a multiple of 128, a 4-bit integer or fp8 weight, up to
+    48 rows - 64 when K is a multiple of 256 and the output length one of 64 - and more than one row.  What differs
+    between the two branches here is what it is in the reference: batch_forward takes x in the dtype it has (a
+    float32 x stays float32), forward_new at more than one row computes in half precision.  The kernels behind
+    both are chosen by the row count alone (up to 16 rows one pass of the streaming kernel, then the ring kernel,
+    then the tiled GEMM)."""
     batch_size = x.shape[0]
-    return (x.dtype in (torch.float, torch.half, torch.bfloat16)
-            and x.shape[1] % 128 == 0
-            and 1 < batch_size <= 16
-            and qtype in (SYM_INT4, ASYM_INT4, SYM_INT8, NF4, FP8E4))
+    hard_condition = (
+        x.dtype in (torch.float, torch.half)
+        and x.shape[1] % 128 == 0
+        and qtype in (SYM_INT4, ASYM_INT4, FP8E5, FP8E4)
+        and (batch_size <= 48 or (batch_size <= 64 and x.shape[1] % 256 == 0 and output_len % 64 == 0))
+    )
+    return hard_condition and batch_size > 1
 
 
 # ------------------------------------------------------------------ device ops
@@ -268,7 +276,7 @@ def forward_new(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int, 
 
 
 def batch_forward(x: torch.Tensor, w: torch.Tensor, qtype: int, output_size: int = None, layout: int = None):
-    """xe_batch.batch_forward: same product, 1 < M <= 16 (one pass over the weights).  The reference hands it
+    """xe_batch.batch_forward: same product for the row counts of use_batch_forward.  The reference hands it
     x in the dtype it has (low_bit_linear.py:657-659), so a float32 x stays fp32."""
     if output_size is None:
         k = x.shape[1]

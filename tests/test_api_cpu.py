@@ -166,10 +166,18 @@ def test_forward_of_an_empty_activation():
 
 
 def test_use_batch_forward_window():
+    """The reference's predicate (low_bit_linear.py:272-307) on a device outside its per-device clauses."""
     x = torch.zeros(4, 256, dtype=torch.half)
     assert use_batch_forward(x, 2, 64) and not use_batch_forward(x[:1], 2, 64)
-    assert not use_batch_forward(torch.zeros(32, 256, dtype=torch.half), 2, 64)
+    assert use_batch_forward(torch.zeros(48, 128, dtype=torch.half), 2, 48)
+    assert not use_batch_forward(torch.zeros(49, 128, dtype=torch.half), 2, 64)         # 49..64 rows need K % 256 == 0
+    assert use_batch_forward(torch.zeros(64, 256, dtype=torch.float), 3, 128)
+    assert not use_batch_forward(torch.zeros(64, 256, dtype=torch.half), 2, 96)         # ... and out_len % 64 == 0
+    assert not use_batch_forward(torch.zeros(65, 256, dtype=torch.half), 2, 64)
     assert not use_batch_forward(torch.zeros(4, 192, dtype=torch.half), 2, 64)
+    assert not use_batch_forward(torch.zeros(4, 256, dtype=torch.bfloat16), 2, 64)      # float32 and half only
+    assert use_batch_forward(x, Q["fp8_e4m3"], 64)
+    assert not use_batch_forward(x, Q["sym_int8"], 64) and not use_batch_forward(x, Q["nf4"], 64)
 
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU failure mode")

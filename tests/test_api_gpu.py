@@ -373,7 +373,9 @@ def test_lowbitlinear_float32_input_follows_the_reference_rules():
         lin.weight = FP4Params(w.clone(), qtype=Q["sym_int4"])
         return lin.to("cuda")
     big = 3.0e5                                                            # overflows fp16
-    for rows, conv, stays_fp32 in ((1, True, True), (4, True, True), (40, True, False), (40, False, True)):
+    # (up to 48 rows, 64 here with K % 256 == 0 and out_len % 64 == 0, are the small-batch range: :272-307)
+    for rows, conv, stays_fp32 in ((1, True, True), (4, True, True), (40, True, True), (64, True, True), (65, True, False),
+                                   (65, False, True)):
         x = torch.randn(rows, 256) * (big if stays_fp32 else 1.0)
         y = layer(conv)(x.cuda())
         assert y.dtype == torch.float32 and torch.isfinite(y).all()
