@@ -318,14 +318,14 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
         for (int t = 0; t < U; t++) {
             const int g = gw + t < G ? gw + t : G - 1;
             rw[t] = 1.0f;
-            if constexpr (MOE == 2) load_tile<QT>(moe_tile(g, rw[t]), lane, r, tr[t]);
-            else load_tile<QT>(wrow + (int64_t)g * F::TILE_BYTES, lane, r, tr[t]);
+            if constexpr (MOE == 2) load_tile<QT, true>(moe_tile(g, rw[t]), lane, r, tr[t]);
+            else load_tile<QT, true>(wrow + (int64_t)g * F::TILE_BYTES, lane, r, tr[t]);
         }
         if constexpr (DUAL) {
 #pragma unroll
             for (int t = 0; t < U; t++) {
                 const int g = gw + t;
-                load_tile<QT>(wrow2 + (int64_t)(g < G ? g : G - 1) * F::TILE_BYTES, lane, r, tr[U + t]);
+                load_tile<QT, true>(wrow2 + (int64_t)(g < G ? g : G - 1) * F::TILE_BYTES, lane, r, tr[U + t]);
             }
         }
 #pragma unroll
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const AT *__restrict__ 
 #pragma unroll
             for (int t = 0; t < U; t++) {
                 const int g = gw + t < G ? gw + t : G - 1;
-                load_tile<QT>(wrow + ((int64_t)wi * G + g) * F::TILE_BYTES, lane, r, tr[wi * U + t]);
+                load_tile<QT, true>(wrow + ((int64_t)wi * G + g) * F::TILE_BYTES, lane, r, tr[wi * U + t]);
             }
 
         __builtin_amdgcn_sched_barrier(0);
