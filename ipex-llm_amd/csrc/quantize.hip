@@ -26,6 +26,13 @@ template <int W> __device__ inline float group_min(float v) {
 }
 
 // Signed value of the FIRST element with the largest magnitude in the block.
+// four floats of the source, which is read once: a nontemporal load
+__device__ inline float4 stream4(const float *p) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const f4 v = __builtin_nontemporal_load((const f4 *)p);
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+
 template <int W> __device__ inline float group_first_absmax_signed(const float4 &v, int lane_in_block) {
     float amax = 0.0f, mx = 0.0f;
     const float e[4] = {v.x, v.y, v.z, v.w};
@@ -128,7 +135,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__
     const int64_t blk = t / LPB;
     const int lib = (int)(t % LPB);
     if (blk >= n_blocks) return;                         // whole LPB-groups leave together
-    const float4 v = *(const float4 *)(src + blk * F::QK + lib * 4);
+    const float4 v = stream4(src + blk * F::QK + lib * 4);
 
     uint32_t hdr, mine;
     block_codes<QT>(v, lib, hdr, mine, mids);
@@ -183,7 +190,7 @@ __global__ __launch_bounds__(256) void quantize_tiled_kernel(const float *__rest
         for (int ps = 0; ps < PASSES; ps++) {
             int col = ps * 256 + lane * 4;
             col = col < nt * TILE_COLS ? col : 0;                    // past the strip: a valid re-read, not stored
-            v[i][ps] = *(const float4 *)(src + (row0 + wave * 4 + i) * K + (int64_t)t0 * TILE_COLS + col);
+            v[i][ps] = stream4(src + (row0 + wave * 4 + i) * K + (int64_t)t0 * TILE_COLS + col);
         }
 #pragma unroll
     for (int i = 0; i < 4; i++)
