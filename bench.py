@@ -37,7 +37,7 @@ LLAMA2_7B = [("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096
              ("gate", 11008, 4096), ("up", 11008, 4096), ("down", 4096, 11008)]
 N_LAYERS = 32
 # HBM bytes per launch of the metric's GEMV from rocprofv3 counters (FETCH_SIZE x 1.9993 + WRITE_SIZE)
-GEMV_TRAFFIC = {"bytes": 25500865, "source": "profiles/gemv_sym_int4_f16_N11008_K4096_M1.md (counter run, not this run)"}
+GEMV_TRAFFIC = {"bytes": 25492716, "source": "profiles/gemv_sym_int4_f16_N11008_K4096_M1.md (counter run, not this run)"}
 
 
 def blob_bytes(n, k, qtype=SYM_INT4):
