@@ -25,6 +25,9 @@ __global__ __launch_bounds__(64 * WAVES) void floor_read_kernel(const u32x4 *__r
         if constexpr (FLAGS & FLOOR_NT) v[i] = __builtin_nontemporal_load(src + idx);
         else v[i] = src[idx];
     }
+    // (left alone the compiler issues two loads, consumes the first and only then issues the next: the wave
+    // then has two loads in flight instead of U)
+    __builtin_amdgcn_sched_barrier(0);
     uint32_t a = 0;
 #pragma unroll
     for (int i = 0; i < U; i++) a ^= v[i][0] ^ v[i][1] ^ v[i][2] ^ v[i][3];
