@@ -116,6 +116,23 @@ def test_gemv_tiled_against_oracle(qtype, dtype, m):
 
 
 @pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+def test_gemv_four_tiles_per_wave_against_oracle(qtype, dtype, m):
+    """Up to four rows of x on a weight with at least 8192 rows and K <= 4096 take the shape of the kernel with four
+    tiles per wave (the metric's [11008 x 4096] does): K = 640 leaves a wave's last tiles past the end."""
+    n, k = 8192, 640
+    w = weights(4400 + qtype, (n, k))
+    x = acts(4500 + m, m, k, dtype)
+    blob_np = orc.quantize(w, qtype)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n, fn="gemv")
+    y_exact = orc.mul_mat_exact(blob_np, x.float().numpy(), (n, k), qtype)
+    assert np.isfinite(y).all()
+    assert np.abs(y - y_exact).max() <= _tol(dtype, qtype) * np.abs(y_exact).max()
+
+
+@pytest.mark.parametrize("qtype", ALL)
 @pytest.mark.parametrize("waves", [1, 3, 16])
 def test_gemv_any_wave_count(qtype, waves):
     n, k = 32, 896      # 7 tiles along K: uneven split over the waves
