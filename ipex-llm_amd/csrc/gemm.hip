@@ -97,17 +97,21 @@ int gemm_splits(int M, int N, int K, size_t ws_bytes, int qtype) {
     const size_t tiles = (size_t)((M + GM - 1) / GM) * (size_t)((N + GN - 1) / GN);
     const size_t per_split = tiles * GM * GN * sizeof(float);     // whole tiles: partial sums keep the tile layout
     const int G = K / TILE_COLS;
+    const double unsplit_t = gemm_time_us(M, N, K, 1, qtype);
     int best = 1;
-    double best_t = gemm_time_us(M, N, K, 1, qtype);
+    double best_t = unsplit_t;
     for (int s = 2; s <= 16 && s * 2 <= G; s++) {
         if ((size_t)s * per_split > ws_bytes) break;
         const double t = gemm_time_us(M, N, K, s, qtype);
-        if (t < 0.95 * best_t) {                                  // a split must pay clearly
+        if (t < best_t) {
             best = s;
             best_t = t;
         }
     }
-    return best;
+    // Splitting must pay clearly against not splitting - not each count against the one before it: with that rule
+    // [4096 x 4096] at M = 512 stopped at two splits (31.0 us) where three take 29.5, and [4096 x 11008] at three
+    // (55.1) where four take 53.8.
+    return best_t < 0.95 * unsplit_t ? best : 1;
 }
 
 // How many column tiles (256 weight rows each) the tall form takes, from the left: whole rounds of one
