@@ -95,6 +95,8 @@ def main():
     ap.add_argument("--floor-only", action="store_true",
                     help="run the serialized [11008 x 4096] GEMV loop next to what launches that only READ the same bytes "
                          "cost in the same chain (libstream_floor.so: an empty kernel, twelve read patterns)")
+    ap.add_argument("--llama3-70b-only", action="store_true",
+                    help="run only the Llama-3-70B linear set (nf4 and sym_int8, bf16, M = 1, 16, 1024)")
     ap.add_argument("--moe-only", action="store_true",
                     help="run only the Mixtral expert FFN legs (fp8_e4m3, 512 tokens top-2, and one token)")
     args = ap.parse_args()
@@ -265,6 +267,10 @@ def main():
 
     if args.moe_only:
         print(json.dumps(moe_legs()))
+        return
+
+    if args.llama3_70b_only:
+        print(json.dumps(other_configs(ggml, torch, gen, dev, None, capture, time_graph, stream, new_weight, only_70b=True)))
         return
 
     # ---- synthetic weights: N(0, 0.02) with 0.1 % outliers at +-0.5, quantized on the GPU
@@ -511,7 +517,7 @@ def main():
     print(json.dumps(out))
 
 
-def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, new_weight):
+def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, new_weight, only_70b=False):
     """The parity-test configurations of BASELINE.json timed once each (not the headline): configs[2] prefill
     and configs[3] Llama-3-70B shapes in nf4 / sym_int8."""
     res = {}
@@ -541,16 +547,17 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
         out["launches"] = len(mods)
         return out
 
-    # configs[2]: one layer's 7 linears at M = 512 / 2048, sym_int4 and asym_int4, fp16
-    sym = [(n, k, b) for _, n, k, b in layer0]
-    asym = [(n, k, new_weight(n, k, QT["asym_int4"], 0.02, outliers=True)) for n, k, _ in sym]
-    for name, mods in (("sym_int4", sym), ("asym_int4", asym)):
-        for m in (512, 2048):
-            res[f"prefill_layer_{name}_M{m}"] = leg(mods, QT[name], ggml.DT_F16, torch.float16, m, 5, True)
-    # the same layer at serving batch sizes (one decode token per sequence)
-    for m in (32, 64, 128):
-        res[f"batched_decode_layer_sym_int4_M{m}"] = leg(sym, QT["sym_int4"], ggml.DT_F16, torch.float16, m, 10, False)
-    del asym
+    if not only_70b:
+        # configs[2]: one layer's 7 linears at M = 512 / 2048, sym_int4 and asym_int4, fp16
+        sym = [(n, k, b) for _, n, k, b in layer0]
+        asym = [(n, k, new_weight(n, k, QT["asym_int4"], 0.02, outliers=True)) for n, k, _ in sym]
+        for name, mods in (("sym_int4", sym), ("asym_int4", asym)):
+            for m in (512, 2048):
+                res[f"prefill_layer_{name}_M{m}"] = leg(mods, QT[name], ggml.DT_F16, torch.float16, m, 5, True)
+        # the same layer at serving batch sizes (one decode token per sequence)
+        for m in (32, 64, 128):
+            res[f"batched_decode_layer_sym_int4_M{m}"] = leg(sym, QT["sym_int4"], ggml.DT_F16, torch.float16, m, 10, False)
+        del asym
     # configs[3]: Llama-3-70B linear set (q, k, v, gate, up, down), bf16
     shapes70 = [(8192, 8192), (1024, 8192), (1024, 8192), (28672, 8192), (28672, 8192), (8192, 28672)]
     for name in ("nf4", "sym_int8"):
