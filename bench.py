@@ -547,6 +547,12 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
         out["launches"] = len(mods)
         return out
 
+    def merged_qkv(mods):
+        """The first three weights (q, k, v: same K) as one: the tile rows of a merged weight follow each other in
+        the tiled layout, so the blobs concatenate."""
+        (nq, k, bq), (nk, _, bk), (nv, _, bv) = mods[:3]
+        return [(nq + nk + nv, k, torch.cat([bq, bk, bv]))] + list(mods[3:])
+
     if not only_70b:
         # configs[2]: one layer's 7 linears at M = 512 / 2048, sym_int4 and asym_int4, fp16
         sym = [(n, k, b) for _, n, k, b in layer0]
@@ -554,6 +560,10 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
         for name, mods in (("sym_int4", sym), ("asym_int4", asym)):
             for m in (512, 2048):
                 res[f"prefill_layer_{name}_M{m}"] = leg(mods, QT[name], ggml.DT_F16, torch.float16, m, 5, True)
+        # as a converted model runs the layer: q | k | v are one weight of [12288 x 4096] (merge_qkv), five launches
+        for m in (512, 2048):
+            res[f"prefill_layer_sym_int4_M{m}_merged_qkv"] = leg(merged_qkv(sym), QT["sym_int4"], ggml.DT_F16,
+                                                                 torch.float16, m, 5, True)
         # the same layer at serving batch sizes (one decode token per sequence)
         for m in (32, 64, 128):
             res[f"batched_decode_layer_sym_int4_M{m}"] = leg(sym, QT["sym_int4"], ggml.DT_F16, torch.float16, m, 10, False)
@@ -564,7 +574,12 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
         mods = [(n, k, new_weight(n, k, QT[name], 0.015)) for n, k in shapes70]
         for m in (1, 16, 1024):
             res[f"llama3_70b_{name}_M{m}"] = leg(mods, QT[name], ggml.DT_BF16, torch.bfloat16, m, 5 if m > 16 else 20, m > 16)
-        del mods
+        # q | k | v as one weight of [10240 x 8192], four launches
+        mq = merged_qkv(mods)
+        for m in (1, 16, 1024):
+            res[f"llama3_70b_{name}_M{m}_merged_qkv"] = leg(mq, QT[name], ggml.DT_BF16, torch.bfloat16, m,
+                                                            5 if m > 16 else 20, m > 16)
+        del mods, mq
     return res
 
 
