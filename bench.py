@@ -547,6 +547,28 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
         out["launches"] = len(mods)
         return out
 
+    def fused_mlp_leg(mods, qtype, dt, tdt, m, reps):
+        """mods = [qkv, o, gate, up, down]: gate and up go out as one lowbit_mlp_forward launch (SiLU and the product in
+        its epilogue; the FLOP counted are the linears' alone, as in the other legs)."""
+        (nq, kq, bq), (no, ko, bo), (ng, kg, bg), (_, _, bu), (nd, kd, bd) = mods
+        x = torch.randn((m, kq), generator=gen, device=dev, dtype=torch.float32).to(tdt)
+        ys = [torch.empty((m, n), dtype=tdt, device=dev) for n in (nq, no, ng, nd)]
+        ws_bytes = max(16, max(ggml.lowbit_workspace_bytes(m, n, k) for n, k, _ in mods))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+        def run():
+            st = stream()
+            for (n, k, blob), xin, y in (((nq, kq, bq), x, ys[0]), ((no, ko, bo), x, ys[1])):
+                ggml.lowbit_forward_ws(xin.data_ptr(), blob.data_ptr(), y.data_ptr(), qtype, ggml.LAYOUT_TILED, dt, m, n, k,
+                                       ws.data_ptr(), ws_bytes, st)
+            ggml.lowbit_mlp_forward(x.data_ptr(), bg.data_ptr(), bu.data_ptr(), ys[2].data_ptr(), qtype, dt, m, ng, kg, 0, st)
+            ggml.lowbit_forward_ws(ys[2].data_ptr(), bd.data_ptr(), ys[3].data_ptr(), qtype, ggml.LAYOUT_TILED, dt, m, nd, kd,
+                                   ws.data_ptr(), ws_bytes, st)
+        ms = time_graph(capture(run), reps, 2)
+        out = mfma(sum(2.0 * m * n * k for n, k, _ in mods), ms)
+        out["launches"] = 4
+        return out
+
     def merged_qkv(mods):
         """The first three weights (q, k, v: same K) as one: the tile rows of a merged weight follow each other in
         the tiled layout, so the blobs concatenate."""
@@ -560,10 +582,13 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
         for name, mods in (("sym_int4", sym), ("asym_int4", asym)):
             for m in (512, 2048):
                 res[f"prefill_layer_{name}_M{m}"] = leg(mods, QT[name], ggml.DT_F16, torch.float16, m, 5, True)
-        # as a converted model runs the layer: q | k | v are one weight of [12288 x 4096] (merge_qkv), five launches
+        # as a converted model runs the layer: q | k | v are one weight of [12288 x 4096] (merge_qkv), five launches;
+        # and with gate and up in the fused launch that also applies the activation (lowbit_mlp_forward), four
         for m in (512, 2048):
             res[f"prefill_layer_sym_int4_M{m}_merged_qkv"] = leg(merged_qkv(sym), QT["sym_int4"], ggml.DT_F16,
                                                                  torch.float16, m, 5, True)
+            res[f"prefill_layer_sym_int4_M{m}_merged_qkv_fused_mlp"] = fused_mlp_leg(merged_qkv(sym), QT["sym_int4"], ggml.DT_F16,
+                                                                                 torch.float16, m, 5)
         # the same layer at serving batch sizes (one decode token per sequence)
         for m in (32, 64, 128):
             res[f"batched_decode_layer_sym_int4_M{m}"] = leg(sym, QT["sym_int4"], ggml.DT_F16, torch.float16, m, 10, False)

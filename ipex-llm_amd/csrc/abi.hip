@@ -13,6 +13,8 @@ int launch_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, v
                            int64_t K, int layout, int out_dtype, hipStream_t st);
 int launch_mlp_gemv(const void *x, const void *wg, const void *wu, void *y, int qtype, int act_dtype, int M, int N,
                     int K, int act, hipStream_t st);
+int launch_mlp_gemm(const void *x, const void *wg, const void *wu, void *y, int qtype, int act_dtype, int M, int N, int K,
+                    int act, hipStream_t st);
 int launch_moe_gemv(const void *x, const int32_t *ids, const float *route_w, int slots, int n_exp, const void *gates,
                     const void *ups, const void *downs, void *h, void *y, int qtype, int act_dtype, int hidden,
                     int inter, int act, hipStream_t st);
@@ -215,40 +217,37 @@ int lowbit_gemm_ws(const void *x, const void *w, void *y, int qtype, int layout,
                       stream);
 }
 
-// shapes for which lowbit_forward_ws considers the ring kernel (see forward_any)
-static bool ring_range(int qtype, int64_t M, int64_t N, int64_t K) {
-    const bool small = (double)M * (double)N * (double)K < 3.5e10;
-    if (qtype == LOWBIT_QT_NF4) return small || ((M + 127) / 128) * ((N + 255) / 256) <= 256;
-    // the other formats: up to 64 rows (its 32- and 64-row tiles); beyond that the tiled GEMM with its K split is
-    // level ([1024 x 8192] at M = 96: 19.2 against 18.6 us) or up to 20 % ahead ([2048 x 4096] at M = 192: 18.5
-    // against 22.8 us, [11008 x 4096] at M = 128: 24.8 against 30.2 us)
-    return small && M <= 64;
-}
+// Row counts up to which lowbit_forward_ws considers the ring kernel (its estimate is fitted up to there): the
+// tiled GEMM's half as many dequantizations per MFMA win beyond, except with nf4, whose code-book lookups weigh on
+// the GEMM's tighter loop.
+static bool ring_range(int qtype, int64_t M) { return M <= (qtype == LOWBIT_QT_NF4 ? 2048 : 256); }
 
-size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    if (M <= 16 || N <= 0 || K < 128 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;   // M <= 16: GEMV
-    if (N % 16 || K % 128) return 0;                                                                  // not tileable: GEMV
-    // enough for whichever kernel lowbit_forward_ws may pick for the shape
-    // the query carries no qtype: the most splits and the widest range any format uses
-    int s = 1;
-    for (const int qt : {LOWBIT_QT_SYM_INT4, LOWBIT_QT_SYM_INT8, LOWBIT_QT_NF4}) {
-        const int sq = gemm_splits((int)M, (int)N, (int)K, (size_t)-1, qt);
-        s = sq > s ? sq : s;
-    }
-    const size_t gemm = s > 1 ? split_bytes(M, N, s) : 0;
-    const size_t ring = ring_range(LOWBIT_QT_NF4, M, N, K) ? ring_workspace_bytes((int)M, (int)N, (int)K, 0) : 0;
-    return gemm > ring ? gemm : ring;
-}
-
-// Choice of kernel behind lowbit_forward, by estimated run time (constants measured on MI355X).  The
-// GEMV streams the weights once per 16 rows of x (2.8 TB/s for the 4-bit integer formats to 5.8 TB/s for sym_int8,
-// plus 2.5 us per pass; later passes come partly out of the Infinity Cache).  The MFMA GEMM amortizes the dequantization over 128 x 256 tiles
-// but is latency-bound while its tiles do not fill the machine: a lone row tile of [11008 x 4096] takes
-// 40 us however few rows it holds, where a GEMV pass takes 12 us.  With a workspace the GEMM can split
-// K over more workgroups at the price of writing and re-reading fp32 partial sums, and the ring kernel
-// (32 / 64 / 128-row tiles, units dealt out evenly) covers the batch sizes in between.
+// Choice of kernel behind lowbit_forward: the one with the shortest estimated run time (estimates fitted to
+// measurements on MI355X: 640 combinations of format, weight shape and M = 17 .. 768, every kernel and split count
+// timed on each; the pick is within 1.5 % of the fastest measured one on average, 21 % at worst).
+//   - The GEMV streams the weights once per 16 rows of x: 4.0 TB/s for the 4-bit integer formats, 5.0 for the 8-bit
+//     ones, 3.3 for nf4, a pass of fewer rows up to 1.46 times that, plus 3.5 us per pass, and never shorter than
+//     its workgroups' walk along K (narrow weights leave CUs idle); the whole scaled by 0.9, see ring_time_us.
+//   - The MFMA GEMM amortizes the dequantization over 128 x 256 tiles but is latency-bound while its tiles do not
+//     fill the machine.  With a workspace it can split K over more workgroups at the price of writing and
+//     re-reading fp32 partial sums (gemm_time_us).
+//   - The ring kernel (32 / 64 / 128-row tiles, units dealt out evenly; needs the workspace) covers the batch
+//     sizes in between (ring_time_us).
 enum { PLAN_GEMV = LOWBIT_PLAN_GEMV, PLAN_RING = LOWBIT_PLAN_RING, PLAN_GEMM = LOWBIT_PLAN_GEMM,
        PLAN_GEMM_SPLIT = LOWBIT_PLAN_GEMM_SPLIT };
+
+static double gemv_time_us(int qtype, int64_t M, int64_t N, int64_t K) {
+    const double rate = qtype == LOWBIT_QT_SYM_INT8 || qtype == LOWBIT_QT_FP8_E4M3 ? 5.03e6 : qtype == LOWBIT_QT_NF4 ? 3.31e6 : 3.97e6;
+    const double bytes = (double)lowbit_blob_bytes(qtype, N * K);
+    const double walk_us = (qtype == LOWBIT_QT_NF4 ? 0.09 : 0.07) * (double)(K / 128);
+    double t = 0.0;
+    for (int64_t m = M; m > 0; m -= 16) {
+        const double rows = m < 16 ? (double)m : 16.0;
+        const double stream_us = bytes / (rate * (1.0 + 0.456 * (16.0 - rows) / 16.0));
+        t += (stream_us > walk_us ? stream_us : walk_us) + 3.5;
+    }
+    return 0.9 * t;
+}
 
 // which kernel, and for PLAN_GEMM_SPLIT into how many K splits
 static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, bool have_ws, size_t workspace_bytes,
@@ -256,30 +255,39 @@ static int plan_forward(int qtype, int layout, int64_t M, int64_t N, int64_t K, 
     if (splits_out) *splits_out = 1;
     if (M <= 16 || layout != LOWBIT_LAYOUT_TILED || !y_aligned8) return PLAN_GEMV;            // the MFMA kernels store 8 bytes and more
     if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || K < 128) return PLAN_GEMM;     // reports the error
-    const double passes = (double)((M + 15) / 16);
-    // a pass cannot be shorter than its workgroups' walk along K (narrow weights leave CUs idle)
-    // bytes per microsecond of a 16-row pass, measured per format ([11008 x 4096] / [28672 x 8192]-sized weights, two to
-    // eight passes back to back): the formats with more bytes per weight have less to compute per byte
-    const double gemv_rate = qtype == LOWBIT_QT_SYM_INT8 ? 5.8e6 : qtype == LOWBIT_QT_FP8_E4M3 ? 4.7e6
-                             : qtype == LOWBIT_QT_NF4 ? 3.3e6 : 2.8e6;
-    const double stream_us = (double)lowbit_blob_bytes(qtype, N * K) / gemv_rate, walk_us = (qtype == LOWBIT_QT_NF4 ? 0.14 : 0.10) * (double)(K / 128);
-    const double t_gemv = passes * ((stream_us > walk_us ? stream_us : walk_us) + 2.5);
     const int splits = have_ws ? gemm_splits((int)M, (int)N, (int)K, workspace_bytes, qtype) : 1;
-    const double t_gemm = gemm_time_us((int)M, (int)N, (int)K, splits, qtype);
-    // The ring kernel needs the workspace for its partial tiles; given that, it measured faster than or level with
-    // the tiled GEMM, split or not, up to M = 64 (sym_int4, sym_int8, fp8_e4m3; five shapes from [1024 x 8192] to
-    // [28672 x 8192]: [4096 x 4096] at M = 64, 15.5 against 18.0 us; at M = 128 23.0 against 20.8).  With nf4, whose code-book lookups weigh on the GEMM's tighter loop, it stays ahead at larger M as well
-    // while the GEMM's tiles are no more than one per CU ([11008 x 4096] at M = 256: 47.5 against 59.4 us).  Its
-    // own estimate decides against the GEMV.
-    if (have_ws && ring_range(qtype, M, N, K) &&
-        ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes)
-        return ring_time_us((int)M, (int)N, (int)K, qtype, true) < t_gemv ? PLAN_RING : PLAN_GEMV;
-    if (t_gemv < t_gemm) return PLAN_GEMV;
-    if (splits > 1) {
-        if (splits_out) *splits_out = splits;
-        return PLAN_GEMM_SPLIT;
+    double best_t = gemm_time_us((int)M, (int)N, (int)K, splits, qtype);
+    int best = splits > 1 ? PLAN_GEMM_SPLIT : PLAN_GEMM;
+    if (M <= 128) {                              // (beyond that eight and more passes never win)
+        const double t = gemv_time_us(qtype, M, N, K);
+        if (t < best_t) { best_t = t; best = PLAN_GEMV; }
     }
-    return PLAN_GEMM;
+    if (have_ws && ring_range(qtype, M) && ring_workspace_bytes((int)M, (int)N, (int)K, 0) <= workspace_bytes) {
+        const double t = ring_time_us((int)M, (int)N, (int)K, qtype, true);
+        if (t < best_t) { best_t = t; best = PLAN_RING; }
+    }
+    if (best == PLAN_GEMM_SPLIT && splits_out) *splits_out = splits;
+    return best;
+}
+
+static size_t plan_workspace(int plan, int splits, int64_t M, int64_t N, int64_t K) {
+    if (plan == PLAN_RING) return ring_workspace_bytes((int)M, (int)N, (int)K, 0);
+    if (plan == PLAN_GEMM_SPLIT) return split_bytes(M, N, splits);
+    return 0;
+}
+
+size_t lowbit_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 16 || N <= 0 || K < 128 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;   // M <= 16: GEMV
+    if (N % 16 || K % 128) return 0;                                                                  // not tileable: GEMV
+    // the query carries no qtype: the most that the plan of any format takes when nothing limits it
+    size_t most = 0;
+    for (const int qt : {LOWBIT_QT_SYM_INT4, LOWBIT_QT_ASYM_INT4, LOWBIT_QT_SYM_INT8, LOWBIT_QT_NF4, LOWBIT_QT_FP8_E4M3}) {
+        int splits = 1;
+        const int plan = plan_forward(qt, LOWBIT_LAYOUT_TILED, M, N, K, true, (size_t)-1, true, &splits);
+        const size_t need = plan_workspace(plan, splits, M, N, K);
+        most = need > most ? need : most;
+    }
+    return most;
 }
 
 // What lowbit_forward_ws will use of a workspace of at most max_bytes for this format and shape: the bytes of the
@@ -446,11 +454,15 @@ int lowbit_mlp_forward(const void *x, const void *w_gate, const void *w_up, void
     if (int rc = check_mm("lowbit_mlp_forward", x, w_gate, y, qtype, LOWBIT_LAYOUT_TILED, act_dtype, M, N, K)) return rc;
     if (act != LOWBIT_ACT_SILU && act != LOWBIT_ACT_GELU)
         return fail(LOWBIT_EARG, "lowbit_mlp_forward: activation must be LOWBIT_ACT_SILU or LOWBIT_ACT_GELU");
-    if (M > 4) return fail(LOWBIT_ESIZE, "lowbit_mlp_forward: M must be at most 4 (decode)");
     if (M * N == 0) return 0;
     if (K == 0) return fail(LOWBIT_ESHAPE, "lowbit_mlp_forward: K == 0");
     if (!w_up || !aligned16(w_up)) return fail(LOWBIT_EARG, "lowbit_mlp_forward: null or misaligned pointer");
-    return check_launch(launch_mlp_gemv(x, w_gate, w_up, y, qtype, act_dtype, (int)M, (int)N, (int)K, act,
+    // up to 4 rows (decode): the streaming kernel; more: the fused gate/up form of the tiled MFMA GEMM
+    if (M <= 4)
+        return check_launch(launch_mlp_gemv(x, w_gate, w_up, y, qtype, act_dtype, (int)M, (int)N, (int)K, act,
+                                            (hipStream_t)stream), "lowbit_mlp_forward");
+    if (((uintptr_t)y) & 7) return fail(LOWBIT_EARG, "lowbit_mlp_forward: y must be 8-byte aligned");
+    return check_launch(launch_mlp_gemm(x, w_gate, w_up, y, qtype, act_dtype, (int)M, (int)N, (int)K, act,
                                         (hipStream_t)stream), "lowbit_mlp_forward");
 }
 

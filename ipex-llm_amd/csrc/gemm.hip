@@ -58,15 +58,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 // partly filled round changes nothing (688 tiles: 161 us either way) or loses 2-6 %.
 static bool half_tiles(int M, int64_t tiles, int n_cus) { return M > GM / 2 && tiles * 8 <= (int64_t)n_cus * 3; }
 
-// Estimated run time in microseconds of the GEMM with K split `splits` ways (1 = no split), fitted to measurements on
-// MI355X (sym_int4 fp16, eight weight shapes from [1024 x 8192] to [28672 x 8192], M = 96 .. 1024, 1 .. 8 splits,
-// each launch on weights it has not just read; the fit is within 8 % rms, and the split it picks within 3 % of the
-// best measured one on average, 13 % at worst): a workgroup takes 1.0 us per 128-column step on an otherwise idle
-// machine and 3.3 us when every CU holds two (the clock drops and the memory system fills as more CUs work); launch,
-// prologue and epilogue come to 9.5 us; a workgroup's fp32 partial tile costs 0.035 us to write and sum.  The formats
-// with more work per weight take longer per step (per step of a launch of a few dozen tiles, without a split:
-// sym_int4 1.03 us, fp8_e4m3 1.30, sym_int8 1.47, nf4 - in the register-staged form that it uses up to one workgroup
-// per CU - 2.7).
+// Estimated run time in microseconds of the 128-row GEMM with K split `splits` ways (1 = no split), fitted to
+// measurements on MI355X: 40 weight shapes from [1024 x 8192] to [28672 x 8192] in all five formats, M = 17 .. 768,
+// 1 .. 16 splits, each launch on weights it has not just read (6200 launches; 9.6 % rms).  What the fit holds:
+//   - a 128-column step takes a workgroup 1.2 us while the launch has up to 128 workgroups, 1.5 us at one per CU,
+//     and 2.1 us and more as soon as two share a CU - a launch of 258 workgroups takes as long as its two shared
+//     CUs ([11008 x 4096] at M = 256: 2 splits = 172 workgroups 36.7 us, 3 splits = 258 workgroups 45.9 us), so the
+//     splits that pay keep the workgroups at or below the number of CUs;
+//   - a row tile that is partly empty skips the MFMAs of its empty 32-row blocks (a sixth of the step per quarter);
+//   - launch, prologue and epilogue come to 2 us, the second launch of a split to 5.4 us, a workgroup's fp32 partial
+//     tile to 0.043 us to write and sum (a quarter of it fixed, the rest by the rows it holds);
+//   - the formats with more work per weight take longer per step: sym_int8 1.30, fp8_e4m3 1.15, nf4 1.30 - 2.48 in
+//     the register-staged form it uses up to one workgroup per CU; half tiles take 0.88 (0.83) of a tile's step.
 double gemm_time_us(int M, int N, int K, int splits, int qtype) {
     const int tiles_m = (M + GM - 1) / GM;
     const double tiles = (double)tiles_m * (double)((N + GN - 1) / GN);
@@ -75,31 +78,28 @@ double gemm_time_us(int M, int N, int K, int splits, int qtype) {
     const int ny = (G + k_steps - 1) / k_steps;
     const bool halves = ny == 1 && qtype != QT_NF4 && half_tiles(M, (int64_t)tiles, 256);   // (nf4: register-staged form)
     const double wgs = tiles * ny * (halves ? 2.0 : 1.0);
-    const double live = wgs < 512.0 ? wgs : 512.0;
-    const double format = qtype == QT_NF4 ? (wgs <= 256.0 ? 2.4 : 1.2) : qtype == QT_SYM_INT8 ? 1.4 : qtype == QT_FP8_E4M3 ? 1.25 : 1.0;
-    // (half a tile repeats the tile's dequantization: the formats that pay most for it gain 3-13 % instead of 15-25 %)
-    const double half = !halves ? 1.0 : (qtype == QT_SYM_INT8 || qtype == QT_FP8_E4M3) ? 0.92 : 0.74;
-    const double step = (1.02 + 2.32 * (live / 512.0) * (live / 512.0)) * half * format;
+    const bool heavy = qtype == QT_SYM_INT8 || qtype == QT_FP8_E4M3;
+    const double format = qtype == QT_NF4 ? (wgs <= 256.0 ? 2.48 : 1.30) : qtype == QT_SYM_INT8 ? 1.30 : qtype == QT_FP8_E4M3 ? 1.15 : 1.0;
+    const double half = !halves ? 1.0 : heavy ? 0.83 : 0.88;
+    const double over128 = wgs > 128.0 ? (wgs - 128.0) / 128.0 : 0.0;
+    const double step = wgs <= 256.0 ? 1.21 + 0.29 * over128 : 2.12 + 0.56 * ((wgs < 512.0 ? wgs : 512.0) - 256.0) / 256.0;
     // workgroups beyond two per CU wait for a slot: the launch lasts as long as the CU that gets most of them
     const double rounds = wgs > 512.0 ? (double)(((int64_t)wgs + 255) / 256) / 2.0 : 1.0;
-    double t = 9.5 + (double)k_steps * step * rounds;
-    // row tiles that are partly empty write fewer partial sums
     const double fill = (double)M / ((double)tiles_m * GM);
-    if (ny > 1) t += 0.035 * (double)ny * tiles * fill;
+    double t = 2.1 + (double)k_steps * step * format * half * rounds * (0.83 + 0.17 * fill);
+    if (ny > 1) t += 5.4 + 0.043 * (double)ny * tiles * (0.24 + 0.76 * fill);
     return t;
 }
 
-// Number of K splits to use for this shape given `ws_bytes` of workspace (1 = none): the fastest by
-// the estimate above among 1 .. 16 splits of at least two K steps that fit the workspace (more than 8 pay on long K
-// with few tiles: fp8_e4m3 [4096 x 14336] at M = 128: 12 splits 33.6 us, 8 splits 35.4; sym_int8 [1024 x 8192]: 16
-// splits 20.0, 8 splits 22.7).
+// Number of K splits to use for this shape given `ws_bytes` of workspace (1 = none): the fastest by the estimate
+// above among 1 .. 16 splits of at least two K steps that fit the workspace.  On the shapes the estimate was fitted
+// to, the split it picks is within 2 % of the best measured one on average.
 int gemm_splits(int M, int N, int K, size_t ws_bytes, int qtype) {
     const size_t tiles = (size_t)((M + GM - 1) / GM) * (size_t)((N + GN - 1) / GN);
     const size_t per_split = tiles * GM * GN * sizeof(float);     // whole tiles: partial sums keep the tile layout
     const int G = K / TILE_COLS;
-    const double unsplit_t = gemm_time_us(M, N, K, 1, qtype);
     int best = 1;
-    double best_t = unsplit_t;
+    double best_t = gemm_time_us(M, N, K, 1, qtype);
     for (int s = 2; s <= 16 && s * 2 <= G; s++) {
         if ((size_t)s * per_split > ws_bytes) break;
         const double t = gemm_time_us(M, N, K, s, qtype);
@@ -108,10 +108,7 @@ int gemm_splits(int M, int N, int K, size_t ws_bytes, int qtype) {
             best_t = t;
         }
     }
-    // Splitting must pay clearly against not splitting - not each count against the one before it: with that rule
-    // [4096 x 4096] at M = 512 stopped at two splits (31.0 us) where three take 29.5, and [4096 x 11008] at three
-    // (55.1) where four take 53.8.
-    return best_t < 0.95 * unsplit_t ? best : 1;
+    return best;
 }
 
 // How many column tiles (256 weight rows each) the tall form takes, from the left: whole rounds of one

@@ -6,5 +6,7 @@ namespace lowbit {
 template int launch_grouped_q<QT_FP8_E4M3>(const void *, const void *const *, const void *const *, void *, const int32_t *, int, int,
                                     int, int, int, int, const GroupedPlan &, float *, hipStream_t);
 
+template int launch_mlp_gemm_q<QT_FP8_E4M3>(const void *, const void *, const void *, void *, int, int, int, int, int, int, bool, hipStream_t);
+
 }  // namespace lowbit
 

@@ -110,6 +110,34 @@ static int launch_grouped_mlp_t(const void *x, const void *const *wg, const void
     return 0;
 }
 
+// The fused gate/up form on a dense gated MLP: y = act(x wg^T) * (x wu^T) for all M rows of x, the two weights
+// given directly (no tables in device memory: see GroupArgs).
+template <int QT, typename AT>
+static int launch_mlp_gemm_t(const void *x, const void *wg, const void *wu, void *y, int M, int N, int K, int act, int waves,
+                             bool one_round, hipStream_t st) {
+    const int tiles_n = (N + GN / 2 - 1) / (GN / 2), G = K / TILE_COLS;
+    const int chunk = grouped_chunk(tiles_n, one_round);
+    const GroupArgs ga = {nullptr, nullptr, nullptr, 1, act, 0, chunk, (const uint8_t *)wu};
+    const int n_wg = grouped_grid((M + GM_TALL - 1) / GM_TALL, tiles_n, chunk);
+    if (waves == 8 || QT == QT_NF4) {                 // (nf4: see launch_grouped_mlp_t)
+        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL, true, true, 8>), dim3(n_wg), dim3(512), 0, st, (const AT *)x,
+                           (const uint8_t *)wg, (AT *)y, M, N, K, 1, ga, G, (float *)nullptr, 0, tiles_n);
+        return 0;
+    }
+    if constexpr (QT != QT_NF4)
+        hipLaunchKernelGGL((gemm_mfma_kernel<QT, AT, true, MB32_TALL, true, true>), dim3(n_wg), dim3(256), 0, st, (const AT *)x,
+                           (const uint8_t *)wg, (AT *)y, M, N, K, 1, ga, G, (float *)nullptr, 0, tiles_n);
+    return 0;
+}
+
+template <int QT>
+int launch_mlp_gemm_q(const void *x, const void *wg, const void *wu, void *y, int dt, int M, int N, int K, int act, int waves,
+                      bool one_round, hipStream_t st) {
+    if (dt == DT_F16) return launch_mlp_gemm_t<QT, _Float16>(x, wg, wu, y, M, N, K, act, waves, one_round, st);
+    if (dt == DT_BF16) return launch_mlp_gemm_t<QT, __bf16>(x, wg, wu, y, M, N, K, act, waves, one_round, st);
+    return -4;
+}
+
 // One weight format: y = x w^T per group, or act(x w^T) * (x w_up^T) when w_up is given.
 template <int QT>
 int launch_grouped_q(const void *x, const void *const *w, const void *const *w_up, void *y, const int32_t *offsets,

@@ -41,6 +41,8 @@ constexpr int GM_TALL = 256, MB32_TALL = GM_TALL / 32;
 // (a few 32-row blocks of x: few MFMAs per weight) cannot cover with its own MFMAs.
 // Grouped mode (mixture-of-experts): rows offsets[e] .. offsets[e+1]-1 of x use the weight w[e]
 // (and w_up[e] in the fused gate/up form); all pointers are device memory.
+// The fused gate/up form also runs a dense gated MLP - one group that holds all M rows - without any table in
+// device memory: offsets == nullptr, the gate weight is the kernel's own `w` argument, the up weight w_up_one.
 struct GroupArgs {
     const int32_t *offsets;
     const uint8_t *const *w;
@@ -50,6 +52,7 @@ struct GroupArgs {
     int split_tail;               // dense 128-row DMA form: the last split_tail tiles of every XCD's share go out as two
                                   // half tiles of 64 rows each, to one workgroup apiece
     int chunk;                    // grouped: column tiles per cell of the tile order (see grouped_tile)
+    const uint8_t *w_up_one;      // fused form without tables (offsets == nullptr): the up weight
 };
 
 // Which row tile of which group, and which column tile, workgroup `b` of a grouped launch works on.
@@ -255,6 +258,12 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
             if (m0 >= M) return;                                                     // (a last row tile of at most 64 rows)
             M = M < m0 + GM / 2 ? M : m0 + GM / 2;                                   // rows past the half are clamped / not stored
         }
+    } else if (DUAL && ga.offsets == nullptr) {
+        // one group of all M rows: the cells are dealt as in a grouped launch, a row tile is 256 rows of x
+        int idx;
+        if (!grouped_cell((M + GM - 1) / GM, tn_cnt, ga.chunk, blockIdx.x, idx, tile_n)) return;     // whole workgroup leaves
+        m0 = idx * GM;
+        w_up = ga.w_up_one;
     } else {
         // every workgroup finds its row tile from the offsets itself
         // (up to 64 groups: lane e also fetches group e's weight pointers while the offsets are on their way)

@@ -362,16 +362,16 @@ def test_kernel_choice_boundaries_are_pinned():
     ms = (1, 16, 17, 32, 64, 128, 256, 511, 512, 1024, 2048)
     #                         1  16  17  32  64 128 256 511 512 1024 2048
     table = {
-        (2, 4096, 4096):   ([G, G, G, G, R, S, S, S, S, S, M], [G, G, G, G, G, M, M, M, M, M, M]),
-        (2, 11008, 4096):  ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
-        (2, 4096, 11008):  ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, M, M, M, M, M, M]),
+        (2, 4096, 4096):   ([G, G, G, G, R, S, S, S, S, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
+        (2, 11008, 4096):  ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
+        (2, 4096, 11008):  ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
         (3, 11008, 4096):  ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
-        (10, 8192, 8192):  ([G, G, R, R, R, R, R, R, R, R, M], [G, G, G, G, G, G, M, M, M, M, M]),
+        (10, 8192, 8192):  ([G, G, R, R, R, R, R, S, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
         (10, 1024, 8192):  ([G, G, R, R, R, R, R, R, R, R, R], [G, G, G, G, G, G, M, M, M, M, M]),
-        (10, 28672, 8192): ([G, G, R, R, R, R, R, M, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
-        (10, 8192, 28672): ([G, G, R, R, R, R, R, R, R, R, M], [G, G, G, G, G, G, M, M, M, M, M]),
-        (8, 28672, 8192):  ([G, G, R, R, R, S, M, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
-        (8, 8192, 28672):  ([G, G, R, R, R, S, S, S, S, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
+        (10, 28672, 8192): ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
+        (10, 8192, 28672): ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
+        (8, 28672, 8192):  ([G, G, R, R, R, S, M, M, M, M, M], [G, G, G, M, M, M, M, M, M, M, M]),
+        (8, 8192, 28672):  ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, M, M, M, M, M, M]),
         (15, 14336, 4096): ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
     }
     for (qtype, n, k), want in table.items():

@@ -27,7 +27,7 @@ def _gelu_tanh(g):
 
 @pytest.mark.parametrize("qtype", ALL)
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m,act", [(1, SILU), (3, GELU), (4, SILU)])
+@pytest.mark.parametrize("m,act", [(1, SILU), (3, GELU), (4, SILU), (5, GELU), (40, SILU), (130, SILU), (300, GELU)])
 def test_mlp_forward_matches_the_exact_gated_product(qtype, dtype, m, act):
     n, k = 304, 640                      # 19 tile rows, K not a multiple of a full round of waves
     wg, wu = weights(9000 + qtype, (n, k)), weights(9100 + qtype, (n, k))
@@ -46,10 +46,12 @@ def test_mlp_forward_rejects_what_it_cannot_fuse():
     n, k = 32, 128
     b = dev_quantize(weights(1, (n, k)), 2, ggml.LAYOUT_TILED)
     x = acts(2, 5, k, torch.float16).cuda()
-    with pytest.raises(RuntimeError, match="at most 4"):
-        mlp_forward_xpu(x, b, b, 5, k, n, SILU, 2)
     with pytest.raises(RuntimeError, match="activation"):
         mlp_forward_xpu(x[:1], b, b, 1, k, n, 7, 2)
+    with pytest.raises(RuntimeError, match="activation"):
+        mlp_forward_xpu(x, b, b, 5, k, n, 7, 2)
+    with pytest.raises(RuntimeError, match="shape"):
+        mlp_forward_xpu(x, b, b, 4, k, n, SILU, 2)
 
 
 class _GatedMlp(nn.Module):
@@ -91,9 +93,15 @@ def test_optimize_model_patches_gated_mlps_and_the_fused_path_agrees(low_bit, ac
             plain = m.down_proj(m.act_fn(m.gate_proj(x1)) * m.up_proj(x1)).float()
             assert fused.shape == plain.shape == (1, 1, 256)
             assert (fused - plain).abs().max() <= 1e-2 * plain.abs().max()
-            y8 = model(x8)                                       # too many rows: the unfused branch
+            y8 = model(x8)                                       # 16 rows: the unfused branch
             assert y8.shape == (2, 8, 256)
             assert torch.equal(y8, m.down_proj(m.act_fn(m.gate_proj(x8)) * m.up_proj(x8)))
+            x80 = torch.randn(2, 40, 256).half().cuda()          # a prefill batch: the fused GEMM
+            assert mlp_fusion_check(x80, Q[low_bit], False) and not mlp_fusion_check(x80.float(), Q[low_bit], False)
+            y80 = model(x80).float()
+            plain = m.down_proj(m.act_fn(m.gate_proj(x80)) * m.up_proj(x80)).float()
+            assert y80.shape == plain.shape == (2, 40, 256)
+            assert (y80 - plain).abs().max() <= 1e-2 * plain.abs().max()
     finally:
         _GatedMlp.__name__ = "_GatedMlp"
 

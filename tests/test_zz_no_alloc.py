@@ -69,7 +69,7 @@ def test_noalloc_equals_forward_ws_on_consecutive_calls():
 
 
 def test_noalloc_rejects_a_shape_beyond_its_scratch():
-    m, n, k = 128, 76800, 1280
+    m, n, k = 768, 8192, 28672
     assert ggml.lowbit_workspace_bytes(m, n, k) > ggml.lowbit_noalloc_scratch_bytes()
     blob = torch.zeros(ggml.lowbit_blob_bytes(Q4_0, n * k), dtype=torch.uint8, device="cuda")
     x = torch.zeros((m, k), dtype=torch.float16, device="cuda")
