@@ -141,11 +141,12 @@ int lowbit_forward(const void *x, const void *w, void *y, int qtype, int layout,
                    int64_t N, int64_t K, void *stream);
 /* Which kernel lowbit_forward (have_workspace = 0) or lowbit_forward_ws (a non-null workspace of
  * workspace_bytes) runs for a shape with an 8-byte aligned y, without running anything: the streaming GEMV in 16-row passes, the ring kernel for batch
- * sizes, or the MFMA GEMM with or without a K split.  Negative for an unknown qtype.  Host arithmetic only. */
+ * sizes, or the MFMA GEMM with or without a K split or in narrow tiles.  Negative for an unknown qtype.  Host arithmetic only. */
 #define LOWBIT_PLAN_GEMV 0
 #define LOWBIT_PLAN_RING 1
 #define LOWBIT_PLAN_GEMM 2
 #define LOWBIT_PLAN_GEMM_SPLIT 3
+#define LOWBIT_PLAN_GEMM_NARROW 4  /* the MFMA GEMM in tiles of 128 weight rows (lowbit_gemm_narrow) */
 /* What lowbit_forward_ws makes use of when the caller can spare at most max_bytes of workspace for this format
  * and shape: the size of the partial tiles of the plan it then picks, 0 when that plan has none.  A caller
  * with a budget asks this instead of capping lowbit_workspace_bytes (which carries no format and returns the most
@@ -161,6 +162,12 @@ int lowbit_gemv(const void *x, const void *w, void *y, int qtype, int layout, in
                 int64_t N, int64_t K, int waves, void *stream);
 int lowbit_gemm(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
                 int64_t N, int64_t K, void *stream);
+/* The MFMA GEMM in tiles of 128 rows of x by 128 weight rows (64 by 128 while those are no more than one per
+ * compute unit) instead of 128 by 256: twice the workgroups for a product whose wider tiles leave compute
+ * units idle, without the partial sums of a K split.  Tiled layout, y 8-byte aligned.  (Same reference
+ * call as lowbit_forward: low_bit_linear.py:657-668.) */
+int lowbit_gemm_narrow(const void *x, const void *w, void *y, int qtype, int layout, int act_dtype, int64_t M,
+                       int64_t N, int64_t K, void *stream);
 
 /* xe_linear.dequantize_rows (python/llm/src/ipex_llm/transformers/embedding.py:218-221; signature
  * xpu_ops.py:59-62): dst[i, :] = dequant(w)[rows[i], :] for i < n_rows, rows = int64 indices in

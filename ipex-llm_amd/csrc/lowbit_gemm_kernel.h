@@ -197,7 +197,10 @@ __device__ inline float gemm_gate_act(float g, int act) {
 // the epilogue stores act(gate) * up.  With eight waves a wave has one 32-row block: its first tile (16 rows) is
 // the gate's, its second the same 16 rows of the up weight, so that both products of an output element still
 // end in the same lane (accumulator i and i + 8).
-template <int QT, typename AT, bool DMA, int MB, bool GROUPED = false, bool DUAL = false, int WAVES = 4>
+// NARROW (dense 128-row DMA form only): 128 weight rows per workgroup instead of 256, one 32-row block per wave -
+// twice the workgroups for a product whose 256-column tiles leave compute units idle, without the partial sums
+// of a K split.
+template <int QT, typename AT, bool DMA, int MB, bool GROUPED = false, bool DUAL = false, int WAVES = 4, bool NARROW = false>
 __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfma_kernel(const AT *__restrict__ x, const uint8_t *__restrict__ w,
                                                         AT *__restrict__ y, int M, int N, int K, int band_m,
                                                         const GroupArgs ga, int k_steps,
@@ -207,8 +210,10 @@ __global__ __launch_bounds__(64 * WAVES, (DMA && MB == 4) ? 2 : 1) void gemm_mfm
     static_assert(MB == 4 || (MB == 8 && DMA), "row tiles of 128 rows, or 256 rows in the DMA form");
     static_assert(!DUAL || (GROUPED && MB == 8), "the fused gate/up form exists for grouped launches of the tall form");
     static_assert(WAVES == 4 || (WAVES == 8 && MB == 8 && DMA), "eight waves: tall form only");
+    static_assert(!NARROW || (DMA && MB == 4 && WAVES == 4 && !GROUPED && !DUAL), "the narrow tile is a dense 128-row DMA form");
     constexpr int MB32 = MB, GM = 32 * MB;            // shadow the 128-row constants of the file
-    constexpr int NB32 = GN / WAVES / 32;             // 32-row weight blocks per wave: 2, or 1 with eight waves
+    constexpr int GN = NARROW ? lowbit::GN / 2 : lowbit::GN;
+    constexpr int NB32 = GN / WAVES / 32;             // 32-row weight blocks per wave: 2, or 1 with eight waves or a narrow tile
     // x block of a K step: 8 * MB32 pieces of 1 KiB (layout below), double buffered
     __shared__ __attribute__((aligned(16))) uint8_t xs[2 * 8 * MB32 * 1024];
     uint8_t *const xs0 = xs, *const xs1 = xs + 8 * MB32 * 1024;

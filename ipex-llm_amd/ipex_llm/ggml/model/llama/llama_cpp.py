@@ -205,9 +205,13 @@ _lib.lowbit_gemm_ring.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_
 _lib.lowbit_gemm_ring.restype = c_int
 
 
+_lib.lowbit_gemm_narrow.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64, c_int64, c_void_p]
+_lib.lowbit_gemm_narrow.restype = c_int
+
+
 _lib.lowbit_forward_plan.argtypes = [c_int, c_int, c_int64, c_int64, c_int64, c_int, c_size_t]
 _lib.lowbit_forward_plan.restype = c_int
-PLAN_GEMV, PLAN_RING, PLAN_GEMM, PLAN_GEMM_SPLIT = 0, 1, 2, 3
+PLAN_GEMV, PLAN_RING, PLAN_GEMM, PLAN_GEMM_SPLIT, PLAN_GEMM_NARROW = 0, 1, 2, 3, 4
 
 
 _lib.lowbit_workspace_bytes_for.argtypes = [c_int, c_int, c_int64, c_int64, c_int64, c_size_t]
@@ -241,6 +245,10 @@ def lowbit_gemm_ws(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, worksp
 def lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, wgs, stream):
     _check(_lib.lowbit_gemm_ring(x, w, y, qtype, layout, act_dtype, m, n, k, workspace, workspace_bytes, wgs,
                                  stream), "lowbit_gemm_ring")
+
+
+def lowbit_gemm_narrow(x, w, y, qtype, layout, act_dtype, m, n, k, stream):
+    _check(_lib.lowbit_gemm_narrow(x, w, y, qtype, layout, act_dtype, m, n, k, stream), "lowbit_gemm_narrow")
 
 
 _lib.lowbit_forward_f32_workspace_bytes.argtypes = [c_int64, c_int64, c_int64]

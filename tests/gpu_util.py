@@ -62,6 +62,8 @@ def dev_matmul(x, blob, qtype, layout, n, fn="forward", waves=0):
         ggml.lowbit_forward(*args, stream())
     elif fn == "gemv":
         ggml.lowbit_gemv(*args, waves, stream())
+    elif fn == "narrow":
+        ggml.lowbit_gemm_narrow(*args, stream())
     else:
         ggml.lowbit_gemm(*args, stream())
     torch.cuda.synchronize()

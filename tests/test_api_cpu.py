@@ -353,7 +353,7 @@ def test_kernel_choice_boundaries_are_pinned():
     (abi.hip, gemm.hip, gemm_ring.hip).  This table pins today's choices for the BASELINE shapes so that a
     re-fit cannot silently route a shape to another kernel: whoever changes a constant re-measures and edits
     the table.  Host arithmetic only (lowbit_forward_plan)."""
-    G, R, M, S = ggml.PLAN_GEMV, ggml.PLAN_RING, ggml.PLAN_GEMM, ggml.PLAN_GEMM_SPLIT
+    G, R, M, S, N = ggml.PLAN_GEMV, ggml.PLAN_RING, ggml.PLAN_GEMM, ggml.PLAN_GEMM_SPLIT, ggml.PLAN_GEMM_NARROW
 
     def plans(qtype, n, k, ms):
         with_ws = [ggml.lowbit_forward_plan(qtype, 1, m, n, k, True, ggml.lowbit_workspace_bytes(m, n, k)) for m in ms]
@@ -362,17 +362,17 @@ def test_kernel_choice_boundaries_are_pinned():
     ms = (1, 16, 17, 32, 64, 128, 256, 511, 512, 1024, 2048)
     #                         1  16  17  32  64 128 256 511 512 1024 2048
     table = {
-        (2, 4096, 4096):   ([G, G, G, G, R, S, S, S, S, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
-        (2, 11008, 4096):  ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
-        (2, 4096, 11008):  ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
-        (3, 11008, 4096):  ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
-        (10, 8192, 8192):  ([G, G, R, R, R, R, R, S, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
-        (10, 1024, 8192):  ([G, G, R, R, R, R, R, R, R, R, R], [G, G, G, G, G, G, M, M, M, M, M]),
-        (10, 28672, 8192): ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, G, M, M, M, M, M, M]),
-        (10, 8192, 28672): ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, G, M, M, M, M, M]),
-        (8, 28672, 8192):  ([G, G, R, R, R, S, M, M, M, M, M], [G, G, G, M, M, M, M, M, M, M, M]),
-        (8, 8192, 28672):  ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, M, M, M, M, M, M]),
-        (15, 14336, 4096): ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, M, M, M, M, M, M, M]),
+        (2, 4096, 4096):   ([G, G, G, G, R, S, S, S, S, N, M], [G, G, G, G, G, N, N, N, N, N, M]),
+        (2, 11008, 4096):  ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, N, N, N, M, M, M, M]),
+        (2, 4096, 11008):  ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, G, N, M, M, M, M]),
+        (3, 11008, 4096):  ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, N, N, N, M, M, M, M]),
+        (10, 8192, 8192):  ([G, G, R, R, R, R, R, S, S, S, M], [G, G, G, G, G, N, N, N, N, N, M]),
+        (10, 1024, 8192):  ([G, G, R, R, R, R, R, R, R, R, R], [G, G, G, G, G, G, N, N, N, N, N]),
+        (10, 28672, 8192): ([G, G, R, R, R, S, S, M, M, M, M], [G, G, G, G, N, N, N, M, M, M, M]),
+        (10, 8192, 28672): ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, N, N, N, N, N, M]),
+        (8, 28672, 8192):  ([G, G, R, R, R, S, M, M, M, M, M], [G, G, N, N, N, N, M, M, M, M, M]),
+        (8, 8192, 28672):  ([G, G, R, R, R, S, S, S, S, S, M], [G, G, G, G, G, N, N, N, N, M, M]),
+        (15, 14336, 4096): ([G, G, R, R, R, S, N, M, M, M, M], [G, G, G, G, N, N, N, M, M, M, M]),
     }
     for (qtype, n, k), want in table.items():
         assert plans(qtype, n, k, ms) == (want[0], want[1]), (qtype, n, k, plans(qtype, n, k, ms))

@@ -205,6 +205,39 @@ def test_gemm_against_oracle(qtype, dtype, m, n, k):
         assert np.abs(y - y_ref).max() <= 1e-2 * np.abs(y_ref).max()
 
 
+# (m, n, k): half tiles with a tail (65 rows: 64 + 1), a weight of one narrow tile and a half, full tiles with an
+# odd number of K steps, three row tiles with a tail of 44 rows, more narrow tiles than the half-tile limit
+NARROW_CASES = [(65, 144, 256), (128, 192, 128), (100, 272, 384), (300, 1008, 1024), (513, 2064, 512)]
+
+
+@pytest.mark.parametrize("qtype", ALL)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", NARROW_CASES)
+def test_gemm_narrow_tiles_against_oracle(qtype, dtype, m, n, k):
+    w = weights(5600 + qtype + m, (n, k))
+    x = acts(5601 + m, m, k, dtype)
+    blob_np = orc.quantize(w, qtype)
+    blob = dev_quantize(w, qtype, TILED)
+    y = dev_matmul(x, blob, qtype, TILED, n, fn="narrow")
+    y_exact = orc.mul_mat_exact(blob_np, x.float().numpy(), (n, k), qtype)
+    assert np.isfinite(y).all()
+    tol = 2e-3 if dtype == torch.float16 else 8e-3
+    assert np.abs(y - y_exact).max() <= tol * np.abs(y_exact).max()
+
+
+def test_gemm_narrow_tiles_at_full_size_agree_with_the_decode_kernel():
+    # [4096 x 4096] at M = 512 and 1024 (256 half tiles; 256 tiles): where lowbit_forward_ws picks this form
+    n = k = 4096
+    w = weights(5610, (n, k))
+    blob = dev_quantize(w, Q4_0, TILED)
+    for m in (512, 1024):
+        x = acts(5611 + m, m, k, torch.float16)
+        y = dev_matmul(x, blob, Q4_0, TILED, n, fn="narrow")
+        rows = [0, 63, 64, 127, 128, m - 1]
+        yv = dev_matmul(x[rows], blob, Q4_0, TILED, n, fn="gemv")
+        assert np.abs(y[rows] - yv).max() <= 2e-3 * np.abs(yv).max()
+
+
 def test_gemm_prefill_shape_sym_and_asym_int4():
     # one Llama-2-7B linear at prefill length: [4096 x 4096], M = 512, fp16 (BASELINE configs[2])
     n = k = 4096

@@ -39,8 +39,8 @@ def _both(x, blob, qtype, n):
 # (qtype, dtype, m, n, k) in call order: a batch-sized product whose tiles are cut along K (partial tiles
 # through the scratch), then a smaller one, then a prefill-sized one that splits K, then one that needs no
 # workspace at all
-CALLS = [(Q4_0, torch.float16, 128, 11008, 4096), (Q4_0, torch.float16, 40, 4096, 1024),
-         (Q8_0, torch.bfloat16, 600, 4096, 2048), (NF4, torch.bfloat16, 100, 528, 2048),
+CALLS = [(Q4_0, torch.float16, 128, 11008, 4096), (Q4_0, torch.float16, 40, 8192, 2048),
+         (Q8_0, torch.bfloat16, 520, 1024, 4096), (NF4, torch.bfloat16, 100, 528, 2048),
          (Q4_0, torch.float16, 4, 1024, 512)]
 
 
