@@ -97,6 +97,8 @@ def main():
                          "cost in the same chain (libstream_floor.so: an empty kernel, twelve read patterns)")
     ap.add_argument("--llama3-70b-only", action="store_true",
                     help="run only the Llama-3-70B linear set (nf4 and sym_int8, bf16, M = 1, 16, 1024)")
+    ap.add_argument("--mlp-only", action="store_true",
+                    help="only the gated MLP at prefill: gate and up as two launches plus the activation, and as one fused launch")
     ap.add_argument("--moe-only", action="store_true",
                     help="run only the Mixtral expert FFN legs (fp8_e4m3, 512 tokens top-2, and one token)")
     args = ap.parse_args()
@@ -264,6 +266,45 @@ def main():
         tok_bytes = 2 * 3 * blobs["w1"][0].numel() + 2 * (hid + 2 * ffn + 2 * ffn + hid)
         res["mixtral_moe_fp8_decode_top2"] = hbm(tok_bytes, ms, kernel="gemv_mfma_kernel<fp8_e4m3,bf16> expert modes, 2 launches per token")
         return res
+
+    def mlp_legs():
+        """The gate and up projections of a Llama-2-7B MLP ([11008 x 4096] each) on a prefill batch, fp16 and bf16:
+        as the reference's modules run them - two products, then SiLU and the product as elementwise kernels (torch's:
+        they are not this library's, and are timed here because the fused launch replaces them) - and as one
+        lowbit_mlp_forward launch.  Six weight pairs per graph replay, so that the weights come from HBM."""
+        import torch.nn.functional as F
+        res = {}
+        n, k = 11008, 4096
+        pairs = [(new_weight(n, k, SYM_INT4, 0.02, outliers=True), new_weight(n, k, SYM_INT4, 0.02, outliers=True)) for _ in range(6)]
+        for tdt, dt, tag in ((torch.float16, ggml.DT_F16, "f16"), (torch.bfloat16, ggml.DT_BF16, "bf16")):
+            for m in (512, 2048):
+                x = torch.randn((m, k), generator=gen, device=dev).to(tdt)
+                g, u, h = (torch.empty((m, n), dtype=tdt, device=dev) for _ in range(3))
+                ws_bytes = max(16, ggml.lowbit_workspace_bytes(m, n, k))
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+                def two():
+                    st = stream()
+                    for a, b in pairs:
+                        for blob, y in ((a, g), (b, u)):
+                            ggml.lowbit_forward_ws(x.data_ptr(), blob.data_ptr(), y.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED, dt, m, n, k,
+                                                   ws.data_ptr(), ws_bytes, st)
+                        torch.mul(F.silu(g), u, out=h)
+
+                def fused():
+                    st = stream()
+                    for a, b in pairs:
+                        ggml.lowbit_mlp_forward(x.data_ptr(), a.data_ptr(), b.data_ptr(), h.data_ptr(), SYM_INT4, dt, m, n, k, 0, st)
+                ms2 = time_graph(capture(two), 10, 2) / len(pairs)
+                ms1 = time_graph(capture(fused), 10, 2) / len(pairs)
+                leg = mfma(2 * 2.0 * m * n * k, ms1, kernel="gemm_mfma_kernel<sym_int4> fused gate/up form, one table-free group")
+                leg["two_launches_plus_activation_ms"] = round(ms2, 4)
+                res[f"prefill_mlp_gate_up_sym_int4_{tag}_M{m}"] = leg
+        return res
+
+    if args.mlp_only:
+        print(json.dumps(mlp_legs()))
+        return
 
     if args.moe_only:
         print(json.dumps(moe_legs()))
@@ -508,6 +549,7 @@ def main():
         extra["prefill_M2048_N11008_K4096"] = prefill_leg(2048)
         extra["quantize_sym_int4_N11008_K4096"] = quantize_leg(5, 2)
         extra.update(other_configs(ggml, torch, gen, dev, layers[0], capture, time_graph, stream, new_weight))
+        extra.update(mlp_legs())
         extra.update(moe_legs())
         out["extra"] = extra
 
