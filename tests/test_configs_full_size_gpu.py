@@ -116,6 +116,34 @@ def test_llama2_7b_prefill_linears(qtype, n, k):
     _linear_case(9200 + qtype + n // 100 + k, qtype, n, k, (512, 2048), torch.float16, 0.02, True)
 
 
+# The gate and up projections of a Llama-2-7B MLP at prefill through the fused launch (lowbit_mlp_forward beyond
+# 4 rows: what a converted model's MLP runs from 32 rows on): SiLU(x Wg^T) * (x Wu^T) against the oracle's exact
+# products of sampled rows, one rounding of the result.
+@pytest.mark.parametrize("qtype,dtype", [(Q4_0, torch.float16), (Q4_1, torch.bfloat16)])
+def test_llama2_7b_prefill_fused_gate_up(qtype, dtype):
+    n, k = 11008, 4096
+    seed = 9250 + qtype
+    wg, wu = _gpu_weight(seed, n, k, 0.02, True), _gpu_weight(seed + 1, n, k, 0.02, True)
+    (bg, fg), (bu, fu) = _quantize_full(wg, qtype), _quantize_full(wu, qtype)
+    rows = _sample(seed + 2, n, N_ROWS)
+    rg, ru = _oracle_rows(wg, fg, qtype, rows), _oracle_rows(wu, fu, qtype, rows)
+    del wg, wu, fg, fu
+    for m in (40, 512, 2048):
+        x = _acts(seed + 3 + m, m, k, dtype)
+        y = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        ggml.lowbit_mlp_forward(x.data_ptr(), bg.data_ptr(), bu.data_ptr(), y.data_ptr(), qtype, DT[dtype], m, n, k, 0, stream())
+        torch.cuda.synchronize()
+        assert not torch.isnan(y).any()
+        m_rows = _sample(seed + 4, m, M_ROWS)
+        xf = x[torch.from_numpy(m_rows).cuda()].float().cpu().numpy()
+        ys = y[torch.from_numpy(m_rows).cuda()][:, torch.from_numpy(rows).cuda()].float().cpu().numpy()
+        g = orc.mul_mat_exact(rg, xf, (len(rows), k), qtype)
+        u = orc.mul_mat_exact(ru, xf, (len(rows), k), qtype)
+        want = g / (1.0 + np.exp(-g)) * u
+        tol = 2e-3 if dtype == torch.float16 else 8e-3
+        assert np.abs(ys - want).max() <= tol * np.abs(want).max(), (qtype, m)
+
+
 # configs[3]: Llama-3-70B linears, nf4 and sym_int8, bf16, M in {1, 16, 1024}; weights N(0, 0.015)
 @pytest.mark.parametrize("qtype", [NF4, Q8_0])
 @pytest.mark.parametrize("n,k", [(8192, 8192), (1024, 8192), (28672, 8192), (8192, 28672)])
