@@ -42,6 +42,22 @@ def test_mlp_forward_matches_the_exact_gated_product(qtype, dtype, m, act):
     assert np.abs(y - want).max() <= tol * np.abs(want).max()
 
 
+def test_mlp_forward_whose_row_tiles_are_a_single_round():
+    # nine row tiles of 256 rows by three column tiles: few enough for one round of workgroups, where a row tile's
+    # column tiles stay on one XCD (the other tile order of the fused launch); the last row tile holds 37 rows
+    m, n, k = 2048 + 37, 272, 256
+    wg, wu = weights(9300, (n, k)), weights(9301, (n, k))
+    x = acts(9302, m, k, torch.float16)
+    bg, bu = dev_quantize(wg, 2, ggml.LAYOUT_TILED), dev_quantize(wu, 2, ggml.LAYOUT_TILED)
+    y = mlp_forward_xpu(x.cuda(), bg, bu, m, k, n, SILU, 2).float().cpu().numpy()
+    xf = x.float().numpy()
+    g = orc.mul_mat_exact(orc.quantize(wg, 2), xf, (n, k), 2)
+    u = orc.mul_mat_exact(orc.quantize(wu, 2), xf, (n, k), 2)
+    want = _silu(g) * u
+    assert np.isfinite(y).all()
+    assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max()
+
+
 def test_mlp_forward_rejects_what_it_cannot_fuse():
     n, k = 32, 128
     b = dev_quantize(weights(1, (n, k)), 2, ggml.LAYOUT_TILED)
