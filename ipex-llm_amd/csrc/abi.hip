@@ -478,8 +478,8 @@ int lowbit_mlp_forward(const void *x, const void *w_gate, const void *w_up, void
     if (M * N == 0) return 0;
     if (K == 0) return fail(LOWBIT_ESHAPE, "lowbit_mlp_forward: K == 0");
     if (!w_up || !aligned16(w_up)) return fail(LOWBIT_EARG, "lowbit_mlp_forward: null or misaligned pointer");
-    // up to 4 rows (decode): the streaming kernel; more: the fused gate/up form of the tiled MFMA GEMM
-    if (M <= 4)
+    // up to 16 rows (decode): the streaming kernel; more: the fused gate/up form of the tiled MFMA GEMM
+    if (M <= 16)
         return check_launch(launch_mlp_gemv(x, w_gate, w_up, y, qtype, act_dtype, (int)M, (int)N, (int)K, act,
                                             (hipStream_t)stream), "lowbit_mlp_forward");
     if (((uintptr_t)y) & 7) return fail(LOWBIT_EARG, "lowbit_mlp_forward: y must be 8-byte aligned");

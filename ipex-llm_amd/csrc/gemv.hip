@@ -580,7 +580,11 @@ static int launch_mlp_t(const void *x, const void *wg, const void *wu, void *y, 
     const AT *xp = (const AT *)x;
     const uint8_t *g = (const uint8_t *)wg, *u = (const uint8_t *)wu;
     if (M <= 2) launch_mfma<QT, AT, 1, 2, 1, true>(xp, g, (AT *)y, M, N, K, 8, st, u, act);
-    else launch_mfma<QT, AT, 1, 2, 2, true>(xp, g, (AT *)y, M, N, K, 8, st, u, act);
+    else if (M <= 4) launch_mfma<QT, AT, 1, 2, 2, true>(xp, g, (AT *)y, M, N, K, 8, st, u, act);
+    // 5 .. 16 rows: one tile of each weight per wave and round with up to 16 waves, as the plain product's
+    // kernels that share x between two tile rows
+    else if (M <= 8) launch_mfma<QT, AT, 2, 1, 2, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
+    else launch_mfma<QT, AT, 4, 1, 4, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
     return 0;
 }
 
@@ -592,7 +596,7 @@ static int launch_mlp_q(const void *x, const void *wg, const void *wu, void *y, 
     return -4;
 }
 
-// y[M, N] = act(x Wg^T) * (x Wu^T), M <= 4, both weights tiled [N, K]
+// y[M, N] = act(x Wg^T) * (x Wu^T), M <= 16, both weights tiled [N, K]
 int launch_mlp_gemv(const void *x, const void *wg, const void *wu, void *y, int qtype, int act_dtype, int M, int N,
                     int K, int act, hipStream_t st) {
     if (M == 0 || N == 0) return 0;

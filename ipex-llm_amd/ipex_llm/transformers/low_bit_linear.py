@@ -329,7 +329,7 @@ def mlp_forward_xpu(x: torch.Tensor, weight1: torch.Tensor, weight2: torch.Tenso
                     state_size: int, output_size: int, act_type: int, qtype: int):
     """xe_linear.mlp_forward_xpu (models/common.py:152-156, xpu_ops.py:34-37):
     act(x @ W1^T) * (x @ W2^T) in one launch; act_type 0 = SiLU, 1 = GELU (tanh form).  Any number of rows:
-    up to 4 run the streaming kernel, more the fused gate/up form of the tiled GEMM (made for prefill batches)."""
+    up to 16 run the streaming kernel, more the fused gate/up form of the tiled GEMM (made for prefill batches)."""
     invalidInputError(x.dim() == 2 and x.shape == (batch_size, state_size) and x.device.type == _ACCEL,
                       "mlp_forward_xpu expects x of shape [batch_size, state_size] on the GPU")
     invalidInputError(ggml.lowbit_tileable(qtype, output_size, state_size),
