@@ -519,7 +519,7 @@ def main():
                 fwd(xs[11008], d["down"], ys["down"], 4096, 11008, st)
         ms5 = time_graph(capture(sweep_merged), max(5, args.steps // 2), 3)
         extra["sweep_merged_qkv_gateup"] = hbm(sweep_bytes(args.m), ms5, launches_per_step=4 * N_LAYERS)
-        if args.m <= 4:
+        if args.m <= 16:
             def mlp(d, st):
                 ggml.lowbit_mlp_forward(xs[4096].data_ptr(), d["gate"].data_ptr(), d["up"].data_ptr(), ym["act"].data_ptr(),
                                         SYM_INT4, ggml.DT_F16, args.m, 11008, 4096, 0, st)
@@ -545,6 +545,26 @@ def main():
             extra["sweep_merged_qkv_fused_mlp"] = hbm(sweep_bytes(args.m), ms7, launches_per_step=4 * N_LAYERS,
                                                       note="what a converted Llama runs per token: qkv_proj, o_proj, "
                                                            "mlp_forward_xpu, down_proj")
+        # the same four launches per layer at M = 4 / 8 (lowbit_mlp_forward fuses gate and up at up to 16 rows)
+        for m in (4, 8):
+            if m == args.m:
+                continue
+            xs2, ys2 = make_io(m)
+            yq = torch.empty((m, 12288), dtype=torch.float16, device=dev)
+            ya = torch.empty((m, 11008), dtype=torch.float16, device=dev)
+
+            def sweep_m_merged_fused():
+                st = stream()
+                for d in merged:
+                    for x, blob, y, n, k in ((xs2[4096], d["qkv"], yq, 12288, 4096), (xs2[4096], d["o"], ys2["o"], 4096, 4096)):
+                        ggml.lowbit_forward(x.data_ptr(), blob.data_ptr(), y.data_ptr(), SYM_INT4, ggml.LAYOUT_TILED, ggml.DT_F16,
+                                            m, n, k, st)
+                    ggml.lowbit_mlp_forward(xs2[4096].data_ptr(), d["gate"].data_ptr(), d["up"].data_ptr(), ya.data_ptr(),
+                                            SYM_INT4, ggml.DT_F16, m, 11008, 4096, 0, st)
+                    ggml.lowbit_forward(xs2[11008].data_ptr(), d["down"].data_ptr(), ys2["down"].data_ptr(), SYM_INT4,
+                                        ggml.LAYOUT_TILED, ggml.DT_F16, m, 4096, 11008, st)
+            ms8 = time_graph(capture(sweep_m_merged_fused), max(5, args.steps // 2), 3)
+            extra[f"sweep_M{m}_merged_qkv_fused_mlp"] = hbm(sweep_bytes(m), ms8, launches_per_step=4 * N_LAYERS)
         del merged
         extra["prefill_M2048_N11008_K4096"] = prefill_leg(2048)
         extra["quantize_sym_int4_N11008_K4096"] = quantize_leg(5, 2)
