@@ -609,7 +609,7 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
         out["launches"] = len(mods)
         return out
 
-    def fused_mlp_leg(mods, qtype, dt, tdt, m, reps):
+    def fused_mlp_leg(mods, qtype, dt, tdt, m, reps, compute_bound=True):
         """mods = [qkv, o, gate, up, down]: gate and up go out as one lowbit_mlp_forward launch (SiLU and the product in
         its epilogue; the FLOP counted are the linears' alone, as in the other legs)."""
         (nq, kq, bq), (no, ko, bo), (ng, kg, bg), (_, _, bu), (nd, kd, bd) = mods
@@ -627,7 +627,8 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
             ggml.lowbit_forward_ws(ys[2].data_ptr(), bd.data_ptr(), ys[3].data_ptr(), qtype, ggml.LAYOUT_TILED, dt, m, nd, kd,
                                    ws.data_ptr(), ws_bytes, st)
         ms = time_graph(capture(run), reps, 2)
-        out = mfma(sum(2.0 * m * n * k for n, k, _ in mods), ms)
+        out = mfma(sum(2.0 * m * n * k for n, k, _ in mods), ms) if compute_bound else \
+            hbm(sum(b.numel() + 2 * m * (n + k) for n, k, b in mods), ms)
         out["launches"] = 4
         return out
 
@@ -654,6 +655,8 @@ def other_configs(ggml, torch, gen, dev, layer0, capture, time_graph, stream, ne
         # the same layer at serving batch sizes (one decode token per sequence)
         for m in (32, 64, 128):
             res[f"batched_decode_layer_sym_int4_M{m}"] = leg(sym, QT["sym_int4"], ggml.DT_F16, torch.float16, m, 10, False)
+            res[f"batched_decode_layer_sym_int4_M{m}_merged_qkv_fused_mlp"] = fused_mlp_leg(merged_qkv(sym), QT["sym_int4"], ggml.DT_F16,
+                                                                                        torch.float16, m, 10, False)
         del asym
     # configs[3]: Llama-3-70B linear set (q, k, v, gate, up, down), bf16
     shapes70 = [(8192, 8192), (1024, 8192), (1024, 8192), (28672, 8192), (28672, 8192), (8192, 28672)]
