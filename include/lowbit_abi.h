@@ -177,8 +177,8 @@ int lowbit_dequantize_rows(const void *w, const int64_t *rows, int64_t n_rows, v
 /* xe_linear.mlp_forward_xpu (python/llm/src/ipex_llm/transformers/models/common.py:145-158; signature
  * xpu_ops.py:34-37): y[M, N] = act(x * Wg^T) .* (x * Wu^T) in one launch, both weights tiled [N, K].
  * Any M (the reference fuses at M == 1 only, models/utils.py:246-259): up to 16 rows run the streaming
- * kernel, more rows the fused gate/up form of the tiled GEMM (y 8-byte aligned, M < 2^24, K < 2^23),
- * which is made for a prefill batch - between 17 and some 30 rows two lowbit_forward calls are faster. */
+ * kernel (one pass over both weights; two passes up to 31 rows while a weight has at most 32 MiB), more
+ * rows the fused gate/up form of the tiled GEMM (y 8-byte aligned, M < 2^24, K < 2^23). */
 int lowbit_mlp_forward(const void *x, const void *w_gate, const void *w_up, void *y, int qtype, int act_dtype,
                        int64_t M, int64_t N, int64_t K, int act, void *stream);
 

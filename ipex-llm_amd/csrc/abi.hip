@@ -478,8 +478,11 @@ int lowbit_mlp_forward(const void *x, const void *w_gate, const void *w_up, void
     if (M * N == 0) return 0;
     if (K == 0) return fail(LOWBIT_ESHAPE, "lowbit_mlp_forward: K == 0");
     if (!w_up || !aligned16(w_up)) return fail(LOWBIT_EARG, "lowbit_mlp_forward: null or misaligned pointer");
-    // up to 16 rows (decode): the streaming kernel; more: the fused gate/up form of the tiled MFMA GEMM
-    if (M <= 16)
+    // up to 16 rows (decode): one pass of the streaming kernel over both weights.  17 .. 31 rows: two passes while
+    // a weight is small enough for that to beat the GEMM form (measured on MI355X at M = 24: sym_int4 [11008 x 4096],
+    // 25 MB a weight, 32.1 against 36.7 us; fp8_e4m3 [14336 x 4096], 61 MB, 53.6 against 47.3; nf4 [28672 x 8192],
+    // 125 MB, 152 against 104).  More rows: the fused gate/up form of the tiled MFMA GEMM.
+    if (M <= 16 || (M < 32 && lowbit_blob_bytes(qtype, N * K) <= ((size_t)32 << 20)))
         return check_launch(launch_mlp_gemv(x, w_gate, w_up, y, qtype, act_dtype, (int)M, (int)N, (int)K, act,
                                             (hipStream_t)stream), "lowbit_mlp_forward");
     if (((uintptr_t)y) & 7) return fail(LOWBIT_EARG, "lowbit_mlp_forward: y must be 8-byte aligned");

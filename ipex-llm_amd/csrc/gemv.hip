@@ -577,14 +577,18 @@ static int launch_mlp_t(const void *x, const void *wg, const void *wu, void *y, 
     // keep the kernel below 80 vector registers, so that a CU holds three workgroups and the 688 workgroups
     // of a [11008 x 4096] pair all run side by side.  With four tiles of each weight the kernel takes 120
     // registers and a third of the workgroups has to wait for a free slot.
-    const AT *xp = (const AT *)x;
     const uint8_t *g = (const uint8_t *)wg, *u = (const uint8_t *)wu;
-    if (M <= 2) launch_mfma<QT, AT, 1, 2, 1, true>(xp, g, (AT *)y, M, N, K, 8, st, u, act);
-    else if (M <= 4) launch_mfma<QT, AT, 1, 2, 2, true>(xp, g, (AT *)y, M, N, K, 8, st, u, act);
-    // 5 .. 16 rows: one tile of each weight per wave and round with up to 16 waves, as the plain product's
-    // kernels that share x between two tile rows
-    else if (M <= 8) launch_mfma<QT, AT, 2, 1, 2, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
-    else launch_mfma<QT, AT, 4, 1, 4, true>(xp, g, (AT *)y, M, N, K, 0, st, u, act);
+    for (int m0 = 0; m0 < M; m0 += 16) {             // one pass over both weights per 16 rows
+        const int mc = (M - m0) < 16 ? (M - m0) : 16;
+        const AT *xp = (const AT *)x + (int64_t)m0 * K;
+        AT *yp = (AT *)y + (int64_t)m0 * N;
+        if (mc <= 2) launch_mfma<QT, AT, 1, 2, 1, true>(xp, g, yp, mc, N, K, 8, st, u, act);
+        else if (mc <= 4) launch_mfma<QT, AT, 1, 2, 2, true>(xp, g, yp, mc, N, K, 8, st, u, act);
+        // 5 .. 16 rows: one tile of each weight per wave and round with up to 16 waves, as the plain product's
+        // kernels that share x between two tile rows
+        else if (mc <= 8) launch_mfma<QT, AT, 2, 1, 2, true>(xp, g, yp, mc, N, K, 0, st, u, act);
+        else launch_mfma<QT, AT, 4, 1, 4, true>(xp, g, yp, mc, N, K, 0, st, u, act);
+    }
     return 0;
 }
 
@@ -596,7 +600,7 @@ static int launch_mlp_q(const void *x, const void *wg, const void *wu, void *y, 
     return -4;
 }
 
-// y[M, N] = act(x Wg^T) * (x Wu^T), M <= 16, both weights tiled [N, K]
+// y[M, N] = act(x Wg^T) * (x Wu^T) in passes of 16 rows, both weights tiled [N, K]
 int launch_mlp_gemv(const void *x, const void *wg, const void *wu, void *y, int qtype, int act_dtype, int M, int N,
                     int K, int act, hipStream_t st) {
     if (M == 0 || N == 0) return 0;

@@ -14,20 +14,13 @@ NF4 = ggml_tensor_qtype["nf4"]
 FP8E4 = ggml_tensor_qtype["fp8_e4m3"]
 
 
-# Up to this many rows the fused launch is the streaming kernel's (one pass over both weights).
-MLP_FUSION_DECODE_ROWS = 16
-# From this many rows on the fused gate/up form of the tiled GEMM beats two products plus the activation as an
-# elementwise kernel (measured on MI355X: level at 32 rows for the integer formats and fp8_e4m3, ahead by 18 % with
-# nf4; at 17 .. 24 rows two passes of the batch-size kernel win).
-MLP_FUSION_PREFILL_ROWS = 32
-
-
 def mlp_fusion_check(x: torch.Tensor, qtype, training: bool) -> bool:
-    """models/utils.py:246-259 of the reference, with this library's limits: the streaming kernel serves up
-    to 16 rows (the reference: exactly 1), the fused GEMM a prefill batch, both in fp16 / bf16 above 4 rows, and
-    every qtype that has a kernel here."""
+    """models/utils.py:246-259 of the reference, with this library's limits: any number of rows (the reference:
+    exactly 1) - the streaming kernel fuses gate and up at decode batch sizes, the tiled GEMM beyond (measured on
+    MI355X against two products plus the activation as elementwise kernels: ahead or level at every row count) - in
+    fp16 / bf16 above 4 rows, and every qtype that has a kernel here."""
     rows = x.numel() // x.size(-1) if x.numel() else 0
-    if rows == 0 or MLP_FUSION_DECODE_ROWS < rows < MLP_FUSION_PREFILL_ROWS:
+    if rows == 0:
         return False
     if rows > 4 and x.dtype not in (torch.float16, torch.bfloat16):
         return False

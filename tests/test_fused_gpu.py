@@ -28,7 +28,7 @@ def _gelu_tanh(g):
 @pytest.mark.parametrize("qtype", ALL)
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m,act", [(1, SILU), (3, GELU), (4, SILU), (5, GELU), (8, SILU), (13, GELU), (16, SILU),
-                                   (17, GELU), (40, SILU), (130, SILU), (300, GELU)])
+                                   (17, GELU), (31, SILU), (32, GELU), (40, SILU), (130, SILU), (300, GELU)])
 def test_mlp_forward_matches_the_exact_gated_product(qtype, dtype, m, act):
     n, k = 304, 640                      # 19 tile rows, K not a multiple of a full round of waves
     wg, wu = weights(9000 + qtype, (n, k)), weights(9100 + qtype, (n, k))
@@ -109,16 +109,17 @@ def test_optimize_model_patches_gated_mlps_and_the_fused_path_agrees(low_bit, ac
             plain = m.down_proj(m.act_fn(m.gate_proj(x1)) * m.up_proj(x1)).float()
             assert fused.shape == plain.shape == (1, 1, 256)
             assert (fused - plain).abs().max() <= 1e-2 * plain.abs().max()
-            x8 = torch.randn(3, 8, 256).half().cuda()
+            x8 = torch.randn(3, 8, 256).cuda()                   # float32 above 4 rows: the unfused branch
             assert not mlp_fusion_check(x8, Q[low_bit], False)
-            y8 = model(x8)                                       # 24 rows: the unfused branch
-            assert y8.shape == (3, 8, 256)
+            y8 = model(x8)
+            assert y8.shape == (3, 8, 256) and y8.dtype == torch.float32
             assert torch.equal(y8, m.down_proj(m.act_fn(m.gate_proj(x8)) * m.up_proj(x8)))
-            x16 = torch.randn(2, 8, 256).half().cuda()           # 16 rows: the streaming kernel's fused launch
-            assert mlp_fusion_check(x16, Q[low_bit], False)
-            y16 = model(x16).float()
-            plain = m.down_proj(m.act_fn(m.gate_proj(x16)) * m.up_proj(x16)).float()
-            assert (y16 - plain).abs().max() <= 1e-2 * plain.abs().max()
+            for rows in (16, 24):                                # the streaming kernel's fused launch, one and two passes
+                xr = torch.randn(rows // 8, 8, 256).half().cuda()
+                assert mlp_fusion_check(xr, Q[low_bit], False)
+                yr = model(xr).float()
+                plain = m.down_proj(m.act_fn(m.gate_proj(xr)) * m.up_proj(xr)).float()
+                assert (yr - plain).abs().max() <= 1e-2 * plain.abs().max()
             x80 = torch.randn(2, 40, 256).half().cuda()          # a prefill batch: the fused GEMM
             assert mlp_fusion_check(x80, Q[low_bit], False) and not mlp_fusion_check(x80.float(), Q[low_bit], False)
             y80 = model(x80).float()
