@@ -99,6 +99,10 @@ def main():
                     help="run only the Llama-3-70B linear set (nf4 and sym_int8, bf16, M = 1, 16, 1024)")
     ap.add_argument("--mlp-only", action="store_true",
                     help="only the gated MLP at prefill: gate and up as two launches plus the activation, and as one fused launch")
+    ap.add_argument("--choice-only", action="store_true",
+                    help="only the check of the kernel choice: lowbit_forward_ws against every kernel it chooses from, "
+                         "timed on the same inputs (--choice-full: the 40 shapes the estimates were fitted on)")
+    ap.add_argument("--choice-full", action="store_true")
     ap.add_argument("--moe-only", action="store_true",
                     help="run only the Mixtral expert FFN legs (fp8_e4m3, 512 tokens top-2, and one token)")
     args = ap.parse_args()
@@ -266,6 +270,79 @@ def main():
         tok_bytes = 2 * 3 * blobs["w1"][0].numel() + 2 * (hid + 2 * ffn + 2 * ffn + hid)
         res["mixtral_moe_fp8_decode_top2"] = hbm(tok_bytes, ms, kernel="gemv_mfma_kernel<fp8_e4m3,bf16> expert modes, 2 launches per token")
         return res
+
+    def choice_check(full):
+        """lowbit_forward_ws against every kernel it chooses from - GEMV passes, the ring kernel, narrow tiles, the
+        GEMM at 1 .. 16 K splits - on the same inputs, each launch on weights it has not just read (several copies
+        per graph replay).  Reports how far the pick lies above the fastest alternative."""
+        F16, BF16 = (torch.float16, ggml.DT_F16), (torch.bfloat16, ggml.DT_BF16)
+        if full:
+            cases = ([(2, F16, sh) for sh in ((11008, 4096), (4096, 4096), (4096, 11008), (12288, 4096), (22016, 4096), (1024, 8192),
+                                             (8192, 8192), (28672, 8192), (8192, 28672), (2048, 2048), (5632, 2048), (2048, 5632),
+                                             (14336, 4096), (4096, 14336))]
+                     + [(2, BF16, sh) for sh in ((11008, 4096), (4096, 4096), (8192, 8192))]
+                     + [(3, F16, sh) for sh in ((11008, 4096), (4096, 4096), (2048, 2048))]
+                     + [(8, BF16, sh) for sh in ((8192, 8192), (1024, 8192), (28672, 8192), (8192, 28672), (10240, 8192))]
+                     + [(8, F16, sh) for sh in ((5632, 2048), (4096, 4096), (11008, 4096))]
+                     + [(15, BF16, sh) for sh in ((14336, 4096), (4096, 14336), (4096, 4096), (6144, 4096))]
+                     + [(10, BF16, sh) for sh in ((28672, 8192), (8192, 8192), (1024, 8192), (8192, 28672), (10240, 8192), (4096, 4096),
+                                                  (11008, 4096), (4096, 11008))])
+            ms = (17, 24, 32, 40, 48, 64, 96, 128, 160, 192, 256, 320, 384, 512, 640, 768, 1024, 1536, 2048)
+        else:
+            cases = [(2, F16, (11008, 4096)), (2, F16, (4096, 4096)), (2, F16, (4096, 11008)), (2, BF16, (4096, 4096)),
+                     (8, BF16, (8192, 8192)), (10, BF16, (8192, 8192)), (15, BF16, (14336, 4096)), (8, F16, (5632, 2048))]
+            ms = (24, 48, 96, 160, 256, 384, 512, 768, 1024, 2048)
+        ws_all = 2 << 30
+        ws = torch.empty(ws_all, dtype=torch.uint8, device=dev)
+        names = {ggml.PLAN_GEMV: "gemv", ggml.PLAN_RING: "ring", ggml.PLAN_GEMM: "gemm", ggml.PLAN_GEMM_SPLIT: "split",
+                 ggml.PLAN_GEMM_NARROW: "narrow"}
+        points = []
+        for qt, (tdt, dt), (n, k) in cases:
+            copies = max(2, min(8, int(400e6 / blob_bytes(n, k, qt))))
+            blobs = [new_weight(n, k, qt, 0.02) for _ in range(copies)]
+            for m in ms:
+                x = torch.randn((m, k), generator=gen, device=dev).to(tdt)
+                y = torch.empty((m, n), dtype=tdt, device=dev)
+                a = (qt, ggml.LAYOUT_TILED, dt, m, n, k)
+
+                def timed(call):
+                    def run():
+                        st = stream()
+                        for b in blobs:
+                            call(b, st)
+                    g = capture(run)
+                    return min(time_graph(g, 4, 2 if i == 0 else 0) for i in range(3)) / copies * 1e3
+                need = max(16, ggml.lowbit_workspace_bytes(m, n, k))
+                alt = {}
+                t_pick = timed(lambda b, st: ggml.lowbit_forward_ws(x.data_ptr(), b.data_ptr(), y.data_ptr(), *a, ws.data_ptr(), need, st))
+                if m <= 128:
+                    alt["gemv"] = timed(lambda b, st: ggml.lowbit_gemv(x.data_ptr(), b.data_ptr(), y.data_ptr(), *a, 0, st))
+                if m <= 256 or qt == 10:
+                    alt["ring"] = timed(lambda b, st: ggml.lowbit_gemm_ring(x.data_ptr(), b.data_ptr(), y.data_ptr(), *a, ws.data_ptr(),
+                                                                            ws_all, 0, st))
+                alt["narrow"] = timed(lambda b, st: ggml.lowbit_gemm_narrow(x.data_ptr(), b.data_ptr(), y.data_ptr(), *a, st))
+                for splits in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16):
+                    tiles = ((m + 127) // 128) * ((n + 255) // 256)
+                    if splits * 2 > k // 128 or splits * tiles * 128 * 256 * 4 > ws_all:
+                        break
+                    alt[f"s{splits}"] = timed(lambda b, st: ggml.lowbit_gemm_ws(x.data_ptr(), b.data_ptr(), y.data_ptr(), *a, ws.data_ptr(),
+                                                                              ws_all, splits, st))
+                best = min(alt, key=alt.get)
+                points.append({"qtype": qt, "act": "f16" if dt == ggml.DT_F16 else "bf16", "N": n, "K": k, "M": m,
+                               "pick": names[ggml.lowbit_forward_plan(qt, ggml.LAYOUT_TILED, m, n, k, True, need)],
+                               "pick_us": round(t_pick, 1), "best": best, "best_us": round(alt[best], 1),
+                               "above_best": round(t_pick / alt[best], 3)})
+            del blobs
+        ratios = sorted(p["above_best"] for p in points)
+        return {"kernel_choice": {"points": len(points), "mean_above_best": round(sum(ratios) / len(ratios), 4),
+                                  "median": ratios[len(ratios) // 2], "more_than_10_percent_above": sum(r > 1.1 for r in ratios),
+                                  "worst": sorted(points, key=lambda p: -p["above_best"])[:8],
+                                  "sum_of_picks_ms": round(sum(p["pick_us"] for p in points) / 1e3, 3),
+                                  "sum_of_bests_ms": round(sum(p["best_us"] for p in points) / 1e3, 3)}}
+
+    if args.choice_only or args.choice_full:
+        print(json.dumps(choice_check(args.choice_full)))
+        return
 
     def mlp_legs():
         """The gate and up projections of a Llama-2-7B MLP ([11008 x 4096] each) on a prefill batch, fp16 and bf16:
